@@ -1,0 +1,135 @@
+/*
+ * ultraattn.h — C ABI of the MI355X (gfx950) block-sparse attention tile library.
+ *
+ * The reference (oliverYoung2001/UltraAttn) has no FFI of its own for this path: its executors
+ * call the Python functions `_flash_attn_forward` / `_flash_attn_backward` of an un-vendored
+ * flash-attention fork and a pure-torch merge.  Each entry point below names the reference
+ * interface it replaces (paths relative to the reference's root).
+ *
+ * Conventions
+ *  - All tensor arguments are DEVICE pointers owned by the caller; the library never allocates,
+ *    frees or synchronises.  Work is enqueued on `stream` (a hipStream_t, NULL = default stream).
+ *  - q, o, dout, dq : [batch, n_qtiles*128, n_heads, 128] bf16, k, v, dk, dv :
+ *    [batch, n_ktiles*128, n_heads, 128] bf16; the innermost (head_dim) axis is contiguous and
+ *    `*_strides` give the element strides of (batch, token, head), each a multiple of 8.
+ *  - lse, delta : [batch, n_heads, n_qtiles*128] fp32, contiguous (the fork's softmax_lse layout,
+ *    orchestrated_attn/orchestrated_attn_impl.py:326 "lse: [mbs, Nh, S]").  Natural log.
+ *  - A tile list is the compacted form of a block mask at 128x128 granularity: CSR over query
+ *    tiles (row_ptr/col_idx/flag, row-major order = search_algo/dependent_graph.py:235-240) and
+ *    the transposed CSC over key tiles.  flag 0 = full tile, 1 = causal tile (key j visible to
+ *    query i iff j <= i on tile-local indices; such tiles sit on the mask's diagonal,
+ *    orchestrated_attn/orchestrated_attn_impl.py:91).  `*_order` is a permutation of the tile
+ *    rows (columns) giving the launch order, longest first.
+ *  - Every function returns 0 (UA_OK) or a negative UA_ERR_* code; ua_strerror() names it.
+ *    No exceptions cross this boundary and nothing aborts.
+ *  - Functions hold no mutable global state and may be called from several host threads on
+ *    different streams.
+ */
+#ifndef ULTRAATTN_H
+#define ULTRAATTN_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define UA_OK 0
+#define UA_ERR_NULL (-1)        /* a required pointer is NULL */
+#define UA_ERR_SHAPE (-2)       /* non-positive or inconsistent sizes */
+#define UA_ERR_UNSUPPORTED (-3) /* head_dim != 128, softmax_scale <= 0, too many partials */
+#define UA_ERR_ALIGN (-4)       /* pointer not 16-byte aligned or stride not a multiple of 8 */
+#define UA_ERR_MASK (-5)        /* block mask holds a value other than 0, 1, 2 */
+#define UA_ERR_LAUNCH (-6)      /* the HIP runtime rejected the launch */
+#define UA_ERR_DEVICE (-7)      /* current device is not a gfx950 GPU */
+
+#define UA_TILE 128        /* rows and columns of one kernel tile */
+#define UA_HEAD_DIM 128    /* the only supported head dimension */
+#define UA_MAX_PARTS 16    /* most partial outputs one ua_merge call combines */
+
+int ua_version(void);
+const char *ua_strerror(int rc);
+
+/* ---- block mask -> active-tile list (host) ------------------------------------------------
+ * Replaces the reference's Python enumeration of Comp_Kernels from a block table:
+ * search_algo/dependent_graph.py:235-263 (row-major order over schedule_table >= 0) with the
+ * refinement rule of search_algo/bsa_config.py:177-213 (complicate_block / complicate).
+ * `block_mask` is a HOST array [n_qblocks, n_kblocks] of Block_Type values
+ * (search_algo/utils.py:140-143: 0 EMPTY, 1 FULL, 2 CAUSAL); every block is refined into
+ * rate x rate tiles (rate = block tokens / 128).  ua_tilelist_size reports the array sizes,
+ * ua_tilelist_build fills caller-allocated HOST arrays:
+ *   row_ptr[n_qtiles+1], col_idx[nnz], flag[nnz]      CSR over query tiles
+ *   col_ptr[n_ktiles+1], row_idx[nnz], cflag[nnz]     CSC over key tiles
+ *   q_order[n_qtiles], k_order[n_ktiles]              longest-first stable orders           */
+int ua_tilelist_size(const uint8_t *block_mask, int n_qblocks, int n_kblocks, int rate,
+                     int64_t *n_qtiles, int64_t *n_ktiles, int64_t *nnz);
+int ua_tilelist_build(const uint8_t *block_mask, int n_qblocks, int n_kblocks, int rate,
+                      int32_t *row_ptr, int32_t *col_idx, uint8_t *flag,
+                      int32_t *col_ptr, int32_t *row_idx, uint8_t *cflag,
+                      int32_t *q_order, int32_t *k_order);
+
+/* Device-side variant: `block_mask` and all outputs are DEVICE arrays (sizes as above, from
+ * ua_tilelist_size on a host copy or an upper bound nnz <= n_qtiles*n_ktiles); `work` is a
+ * device scratch of (n_qtiles + n_ktiles + 2) int32.  Produces the same arrays bit for bit. */
+int ua_tilelist_build_device(const uint8_t *block_mask, int n_qblocks, int n_kblocks, int rate,
+                             int32_t *row_ptr, int32_t *col_idx, uint8_t *flag,
+                             int32_t *col_ptr, int32_t *row_idx, uint8_t *cflag,
+                             int32_t *q_order, int32_t *k_order, int32_t *work, void *stream);
+
+/* ---- forward ------------------------------------------------------------------------------
+ * Replaces the N dense `_flash_attn_forward(q, k, v, dropout_p, softmax_scale, causal=, ...,
+ * out=)` launches of fwd_comp_func (orchestrated_attn/orchestrated_attn_impl.py:320-338; same
+ * call hierarchy_attn/hierarchy_attn_impl.py:40-53) by one launch over the tile list.
+ * Writes o (bf16) and lse (fp32) for every query row; rows without an active tile get o = 0,
+ * lse = -inf.                                                                               */
+int ua_bsa_fwd(const void *q, const void *k, const void *v, void *o, float *lse,
+               const int32_t *row_ptr, const int32_t *col_idx, const uint8_t *flag,
+               const int32_t *q_order,
+               int batch, int n_heads, int n_qtiles, int n_ktiles, int head_dim,
+               const int64_t *q_strides, const int64_t *k_strides, const int64_t *v_strides,
+               const int64_t *o_strides, float softmax_scale, void *stream);
+
+/* ---- backward -----------------------------------------------------------------------------
+ * Replace `_flash_attn_backward(dout, q, k, v, out, softmax_lse, dq, dk, dv, ..., softmax_d=)`
+ * of bwd_comp_func (orchestrated_attn/orchestrated_attn_impl.py:574-597).
+ * ua_bsa_bwd_delta : delta = rowsum(dout * o), the `softmax_d` the reference precomputes.
+ * ua_bsa_bwd_dkdv  : dk, dv for every key row (walks the CSC, no atomics); key rows without an
+ *                    active tile get 0.
+ * ua_bsa_bwd_dq    : dq for every query row (walks the CSR).
+ * lse and delta are the rows' global statistics, the same for every tile of a row
+ * (ring_flash_attn/ring_flash_attn.py:91-108).  Outputs are overwritten, not accumulated. */
+int ua_bsa_bwd_delta(const void *o, const void *dout, float *delta,
+                     int batch, int seqlen_q, int n_heads, int head_dim,
+                     const int64_t *o_strides, const int64_t *do_strides, void *stream);
+int ua_bsa_bwd_dkdv(const void *q, const void *k, const void *v, const void *dout,
+                    const float *lse, const float *delta, void *dk, void *dv,
+                    const int32_t *col_ptr, const int32_t *row_idx, const uint8_t *cflag,
+                    const int32_t *k_order,
+                    int batch, int n_heads, int n_qtiles, int n_ktiles, int head_dim,
+                    const int64_t *q_strides, const int64_t *k_strides, const int64_t *v_strides,
+                    const int64_t *do_strides, const int64_t *dk_strides, const int64_t *dv_strides,
+                    float softmax_scale, void *stream);
+int ua_bsa_bwd_dq(const void *q, const void *k, const void *v, const void *dout,
+                  const float *lse, const float *delta, void *dq,
+                  const int32_t *row_ptr, const int32_t *col_idx, const uint8_t *flag,
+                  const int32_t *q_order,
+                  int batch, int n_heads, int n_qtiles, int n_ktiles, int head_dim,
+                  const int64_t *q_strides, const int64_t *k_strides, const int64_t *v_strides,
+                  const int64_t *do_strides, const int64_t *dq_strides,
+                  float softmax_scale, void *stream);
+
+/* ---- merge of partial outputs ---------------------------------------------------------------
+ * Replaces the chain of `update_out_and_lse` calls (ring_flash_attn/utils.py:38-52, 78-99;
+ * hierarchy_attn/utils.py:16-56; the commented formula at orchestrated_attn/utils.py:120-133)
+ * by one pass over n_parts partials:  LSE = log sum_p exp(lse_p),  O = sum_p exp(lse_p - LSE) O_p
+ * (max-stabilised; a partial with lse = -inf contributes nothing).
+ * o_parts / lse_parts are HOST arrays of n_parts DEVICE pointers: o_parts[p] is a contiguous
+ * [batch, seqlen, n_heads, 128] bf16 tensor, lse_parts[p] a contiguous [batch, n_heads, seqlen]
+ * fp32 tensor; o and lse have the same layouts.  o / lse may alias partial 0.               */
+int ua_merge(const void *const *o_parts, const float *const *lse_parts, int n_parts,
+             void *o, float *lse, int batch, int seqlen, int n_heads, int head_dim, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* ULTRAATTN_H */

@@ -1,0 +1,282 @@
+// Block-sparse flash-attention backward for gfx950 (MI355X): two deterministic kernels that
+// recompute P from the rows' LSE, no atomics.
+//
+//  dkdv_kernel : one workgroup per (key tile, head) walks the CSC column of query tiles.
+//                A wavefront owns 32 key rows; K and V fragments stay in registers, the Q and
+//                dO tiles stream through LDS.  Products (all 32x32x16 bf16 MFMA):
+//                  S [q,key]  = Q K^T          dP[q,key]  = dO V^T
+//                  dV^T[d,key] += dO^T P       dK^T[d,key] += Q^T dS
+//                In the accumulator layout a lane holds one key column, so S / dP blocks
+//                become, after the pointwise step, the B operands of the last two products.
+//  dq_kernel   : one workgroup per (query tile, head) walks the CSR row of key tiles.
+//                A wavefront owns 32 query rows; Q and dO fragments stay in registers, the K
+//                and V tiles stream through LDS:
+//                  S^T[key,q] = K Q^T          dP^T[key,q] = V dO^T
+//                  dQ^T[d,q] += K^T dS^T
+//                Here a lane holds one query column, so lse and delta are per-lane scalars.
+//  P = exp2(scale*log2e*S - lse*log2e);  dS = P * (dP - delta);  dQ, dK are scaled by
+//  softmax_scale on output.
+#include "ua_common.h"
+
+namespace ua {
+
+struct BwdParams {
+  const bf16* q; const bf16* k; const bf16* v; const bf16* dout;
+  const float* lse; const float* delta;
+  bf16* out0; bf16* out1;                  // dkdv: dk, dv; dq: dq, unused
+  const int32_t* ptr; const int32_t* idx; const uint8_t* flag; const int32_t* order;
+  int batch, n_heads, n_qtiles, n_ktiles;
+  Strides3 qs, ks, vs, ds, o0s, o1s;
+  float scale_log2, scale;
+  int heads_per_xcd;
+};
+
+__device__ __forceinline__ void store_acc_t(bf16* row_ptr, const f32x16 (&acc)[4], float mul, int hi) {
+  // acc[mb][4g+j] holds column (32*mb + 8*g + 4*hi + j) of this lane's output row
+#pragma unroll
+  for (int mb = 0; mb < 4; ++mb)
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+      bf16x4 w;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) w[j] = (bf16)(acc[mb][4 * g + j] * mul);
+      *reinterpret_cast<bf16x4*>(row_ptr + 32 * mb + 8 * g + 4 * hi) = w;
+    }
+}
+
+__global__ __launch_bounds__(256, 1) void dkdv_kernel(const BwdParams p) {
+  __shared__ __attribute__((aligned(16))) unsigned char smem[2 * kTileBytes + 2 * kTile * 4];
+  unsigned char* sQ = smem;
+  unsigned char* sdO = smem + kTileBytes;
+  float* sLse = reinterpret_cast<float*>(smem + 2 * kTileBytes);
+  float* sDelta = sLse + kTile;
+
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  const int l32 = lane & 31, hi = lane >> 5;
+  int pos, bh;
+  map_block(blockIdx.x, p.batch * p.n_heads, p.heads_per_xcd, pos, bh);
+  const int kt = p.order[pos];
+  const int b = bh / p.n_heads, h = bh % p.n_heads;
+  const int64_t seq_q = (int64_t)p.n_qtiles * kTile;
+
+  // K, V fragments (B operands): lane holds key row 32*wave + lane%32, d = 16*ks + 8*hi .. +7
+  const int krow = kt * kTile + wave * 32 + l32;
+  const bf16* kp = p.k + b * p.ks.b + (int64_t)krow * p.ks.s + h * p.ks.h + hi * 8;
+  const bf16* vp = p.v + b * p.vs.b + (int64_t)krow * p.vs.s + h * p.vs.h + hi * 8;
+  bf16x8 kf[8], vf[8];
+#pragma unroll
+  for (int ks = 0; ks < 8; ++ks) {
+    kf[ks] = *reinterpret_cast<const bf16x8*>(kp + ks * 16);
+    vf[ks] = *reinterpret_cast<const bf16x8*>(vp + ks * 16);
+  }
+  f32x16 dk[4], dv[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) { dk[i] = f32x16{0}; dv[i] = f32x16{0}; }
+
+  const bf16* qbase = p.q + b * p.qs.b + h * p.qs.h;
+  const bf16* dobase = p.dout + b * p.ds.b + h * p.ds.h;
+  const float* lse_row = p.lse + ((int64_t)b * p.n_heads + h) * seq_q;
+  const float* delta_row = p.delta + ((int64_t)b * p.n_heads + h) * seq_q;
+  const TrLane tr(lane);
+  const int key_l = wave * 32 + l32;
+
+  const int e0 = p.ptr[kt], e1 = p.ptr[kt + 1];
+  for (int e = e0; e < e1; ++e) {
+    const int qt = p.idx[e];
+    const int causal = p.flag[e];
+    if ((unsigned)qt >= (unsigned)p.n_qtiles) continue;
+    __syncthreads();
+    stage_tile<lds_off_u>(sQ, qbase + (int64_t)qt * kTile * p.qs.s, p.qs.s, tid);
+    stage_tile<lds_off_u>(sdO, dobase + (int64_t)qt * kTile * p.ds.s, p.ds.s, tid);
+    if (tid < kTile) {
+      const float l = lse_row[qt * kTile + tid];
+      sLse[tid] = (l == -INFINITY) ? INFINITY : l * kLog2e;   // rows without keys give P = 0
+    } else {
+      sDelta[tid - kTile] = delta_row[qt * kTile + tid - kTile];
+    }
+    __syncthreads();
+
+#pragma unroll 1
+    for (int nb = 0; nb < 4; ++nb) {     // 32 query rows at a time
+      f32x16 s = f32x16{0}, dp = f32x16{0};
+#pragma unroll
+      for (int ks = 0; ks < 8; ++ks) {
+        const bf16x8 aq = lds_read_b128(sQ, lds_off_u(32 * nb + l32, 2 * ks + hi));
+        s = mfma32(aq, kf[ks], s);
+        const bf16x8 ad = lds_read_b128(sdO, lds_off_u(32 * nb + l32, 2 * ks + hi));
+        dp = mfma32(ad, vf[ks], dp);
+      }
+      // element i: query row 32*nb + 8*(i/4) + 4*hi + i%4, key column key_l
+      bf16x8 pb[2], dsb[2];
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        const int q0 = 32 * nb + 8 * g + 4 * hi;
+        const f32x4 l4 = *reinterpret_cast<const f32x4*>(sLse + q0);
+        const f32x4 d4 = *reinterpret_cast<const f32x4*>(sDelta + q0);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const int i = 4 * g + j;
+          float pv = fast_exp2(fmaf(s[i], p.scale_log2, -l4[j]));
+          if (causal && key_l > q0 + j) pv = 0.f;
+          const float dsv = pv * (dp[i] - d4[j]);
+          pb[i >> 3][i & 7] = (bf16)pv;
+          dsb[i >> 3][i & 7] = (bf16)dsv;
+        }
+      }
+#pragma unroll
+      for (int t = 0; t < 2; ++t)
+#pragma unroll
+        for (int mbd = 0; mbd < 4; ++mbd) {
+          const bf16x8 a_do = lds_read_tr_frag<lds_off_u>(sdO, tr, 32 * nb + 16 * t, mbd);
+          dv[mbd] = mfma32(a_do, pb[t], dv[mbd]);
+          const bf16x8 a_q = lds_read_tr_frag<lds_off_u>(sQ, tr, 32 * nb + 16 * t, mbd);
+          dk[mbd] = mfma32(a_q, dsb[t], dk[mbd]);
+        }
+    }
+  }
+  store_acc_t(p.out0 + b * p.o0s.b + (int64_t)krow * p.o0s.s + h * p.o0s.h, dk, p.scale, hi);
+  store_acc_t(p.out1 + b * p.o1s.b + (int64_t)krow * p.o1s.s + h * p.o1s.h, dv, 1.f, hi);
+}
+
+__global__ __launch_bounds__(256, 2) void dq_kernel(const BwdParams p) {
+  __shared__ __attribute__((aligned(16))) unsigned char smem[2 * kTileBytes];
+  unsigned char* sK = smem;
+  unsigned char* sV = smem + kTileBytes;
+
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  const int l32 = lane & 31, hi = lane >> 5;
+  int pos, bh;
+  map_block(blockIdx.x, p.batch * p.n_heads, p.heads_per_xcd, pos, bh);
+  const int qt = p.order[pos];
+  const int b = bh / p.n_heads, h = bh % p.n_heads;
+  const int64_t seq_q = (int64_t)p.n_qtiles * kTile;
+
+  const int qrow = qt * kTile + wave * 32 + l32;
+  const bf16* qp = p.q + b * p.qs.b + (int64_t)qrow * p.qs.s + h * p.qs.h + hi * 8;
+  const bf16* dop = p.dout + b * p.ds.b + (int64_t)qrow * p.ds.s + h * p.ds.h + hi * 8;
+  bf16x8 qf[8], dof[8];
+#pragma unroll
+  for (int ks = 0; ks < 8; ++ks) {
+    qf[ks] = *reinterpret_cast<const bf16x8*>(qp + ks * 16);
+    dof[ks] = *reinterpret_cast<const bf16x8*>(dop + ks * 16);
+  }
+  const float lse_raw = p.lse[((int64_t)b * p.n_heads + h) * seq_q + qrow];
+  const float lse2 = (lse_raw == -INFINITY) ? INFINITY : lse_raw * kLog2e;
+  const float delta = p.delta[((int64_t)b * p.n_heads + h) * seq_q + qrow];
+
+  f32x16 dq[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) dq[i] = f32x16{0};
+  const bf16* kbase = p.k + b * p.ks.b + h * p.ks.h;
+  const bf16* vbase = p.v + b * p.vs.b + h * p.vs.h;
+  const TrLane tr(lane);
+  const int q_l = wave * 32 + l32;
+
+  const int e0 = p.ptr[qt], e1 = p.ptr[qt + 1];
+  for (int e = e0; e < e1; ++e) {
+    const int kt = p.idx[e];
+    const int causal = p.flag[e];
+    if ((unsigned)kt >= (unsigned)p.n_ktiles) continue;
+    __syncthreads();
+    stage_tile<lds_off_u>(sK, kbase + (int64_t)kt * kTile * p.ks.s, p.ks.s, tid);
+    stage_tile<lds_off_k>(sV, vbase + (int64_t)kt * kTile * p.vs.s, p.vs.s, tid);
+    __syncthreads();
+
+#pragma unroll 1
+    for (int mb = 0; mb < 4; ++mb) {     // 32 keys at a time
+      f32x16 s = f32x16{0}, dp = f32x16{0};
+#pragma unroll
+      for (int ks = 0; ks < 8; ++ks) {
+        const bf16x8 ak = lds_read_b128(sK, lds_off_u(32 * mb + l32, 2 * ks + hi));
+        s = mfma32(ak, qf[ks], s);
+        const bf16x8 av = lds_read_b128(sV, lds_off_k(32 * mb + l32, 2 * ks + hi));
+        dp = mfma32(av, dof[ks], dp);
+      }
+      // element i: key 32*mb + 8*(i/4) + 4*hi + i%4, query column q_l
+      bf16x8 dsb[2];
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        const int key = 32 * mb + 8 * (i >> 2) + 4 * hi + (i & 3);
+        float pv = fast_exp2(fmaf(s[i], p.scale_log2, -lse2));
+        if (causal && key > q_l) pv = 0.f;
+        dsb[i >> 3][i & 7] = (bf16)(pv * (dp[i] - delta));
+      }
+#pragma unroll
+      for (int t = 0; t < 2; ++t)
+#pragma unroll
+        for (int mbd = 0; mbd < 4; ++mbd) {
+          const bf16x8 a_k = lds_read_tr_frag<lds_off_u>(sK, tr, 32 * mb + 16 * t, mbd);
+          dq[mbd] = mfma32(a_k, dsb[t], dq[mbd]);
+        }
+    }
+  }
+  store_acc_t(p.out0 + b * p.o0s.b + (int64_t)qrow * p.o0s.s + h * p.o0s.h, dq, p.scale, hi);
+}
+
+static int fill_common(BwdParams& p, const void* q, const void* k, const void* v, const void* dout,
+                       const float* lse, const float* delta, int batch, int n_heads, int n_qtiles,
+                       int n_ktiles, int head_dim, const int64_t* qs, const int64_t* ks,
+                       const int64_t* vs, const int64_t* ds, float softmax_scale) {
+  if (!q || !k || !v || !dout || !lse || !delta || !qs || !ks || !vs || !ds) return UA_ERR_NULL;
+  if (batch <= 0 || n_heads <= 0 || n_qtiles <= 0 || n_ktiles <= 0) return UA_ERR_SHAPE;
+  if ((int64_t)batch * n_heads * n_qtiles > INT32_MAX || (int64_t)batch * n_heads * n_ktiles > INT32_MAX)
+    return UA_ERR_SHAPE;
+  if (head_dim != kHeadDim || !(softmax_scale > 0.f)) return UA_ERR_UNSUPPORTED;
+  if (!aligned16(q) || !aligned16(k) || !aligned16(v) || !aligned16(dout)) return UA_ERR_ALIGN;
+  if (!strides_ok(qs) || !strides_ok(ks) || !strides_ok(vs) || !strides_ok(ds)) return UA_ERR_ALIGN;
+  p.q = (const bf16*)q; p.k = (const bf16*)k; p.v = (const bf16*)v; p.dout = (const bf16*)dout;
+  p.lse = lse; p.delta = delta;
+  p.batch = batch; p.n_heads = n_heads; p.n_qtiles = n_qtiles; p.n_ktiles = n_ktiles;
+  p.qs = {qs[0], qs[1], qs[2]}; p.ks = {ks[0], ks[1], ks[2]};
+  p.vs = {vs[0], vs[1], vs[2]}; p.ds = {ds[0], ds[1], ds[2]};
+  p.scale = softmax_scale; p.scale_log2 = softmax_scale * kLog2e;
+  const int nbh = batch * n_heads;
+  p.heads_per_xcd = (nbh % 8 == 0) ? nbh / 8 : 0;
+  return check_device();
+}
+
+}  // namespace ua
+
+extern "C" int ua_bsa_bwd_dkdv(const void* q, const void* k, const void* v, const void* dout,
+                               const float* lse, const float* delta, void* dk, void* dv,
+                               const int32_t* col_ptr, const int32_t* row_idx, const uint8_t* cflag,
+                               const int32_t* k_order,
+                               int batch, int n_heads, int n_qtiles, int n_ktiles, int head_dim,
+                               const int64_t* q_strides, const int64_t* k_strides, const int64_t* v_strides,
+                               const int64_t* do_strides, const int64_t* dk_strides, const int64_t* dv_strides,
+                               float softmax_scale, void* stream) {
+  using namespace ua;
+  BwdParams p;
+  if (int rc = fill_common(p, q, k, v, dout, lse, delta, batch, n_heads, n_qtiles, n_ktiles, head_dim,
+                           q_strides, k_strides, v_strides, do_strides, softmax_scale)) return rc;
+  if (!dk || !dv || !col_ptr || !k_order || !dk_strides || !dv_strides) return UA_ERR_NULL;
+  if (!aligned16(dk) || !aligned16(dv) || !strides_ok(dk_strides) || !strides_ok(dv_strides)) return UA_ERR_ALIGN;
+  p.out0 = (bf16*)dk; p.out1 = (bf16*)dv;
+  p.o0s = {dk_strides[0], dk_strides[1], dk_strides[2]};
+  p.o1s = {dv_strides[0], dv_strides[1], dv_strides[2]};
+  p.ptr = col_ptr; p.idx = row_idx; p.flag = cflag; p.order = k_order;
+  hipLaunchKernelGGL(dkdv_kernel, dim3((unsigned)(batch * n_heads * n_ktiles)), dim3(256), 0, (hipStream_t)stream, p);
+  return hipGetLastError() == hipSuccess ? UA_OK : UA_ERR_LAUNCH;
+}
+
+extern "C" int ua_bsa_bwd_dq(const void* q, const void* k, const void* v, const void* dout,
+                             const float* lse, const float* delta, void* dq,
+                             const int32_t* row_ptr, const int32_t* col_idx, const uint8_t* flag,
+                             const int32_t* q_order,
+                             int batch, int n_heads, int n_qtiles, int n_ktiles, int head_dim,
+                             const int64_t* q_strides, const int64_t* k_strides, const int64_t* v_strides,
+                             const int64_t* do_strides, const int64_t* dq_strides,
+                             float softmax_scale, void* stream) {
+  using namespace ua;
+  BwdParams p;
+  if (int rc = fill_common(p, q, k, v, dout, lse, delta, batch, n_heads, n_qtiles, n_ktiles, head_dim,
+                           q_strides, k_strides, v_strides, do_strides, softmax_scale)) return rc;
+  if (!dq || !row_ptr || !q_order || !dq_strides) return UA_ERR_NULL;
+  if (!aligned16(dq) || !strides_ok(dq_strides)) return UA_ERR_ALIGN;
+  p.out0 = (bf16*)dq; p.out1 = nullptr;
+  p.o0s = {dq_strides[0], dq_strides[1], dq_strides[2]};
+  p.o1s = p.o0s;
+  p.ptr = row_ptr; p.idx = col_idx; p.flag = flag; p.order = q_order;
+  hipLaunchKernelGGL(dq_kernel, dim3((unsigned)(batch * n_heads * n_qtiles)), dim3(256), 0, (hipStream_t)stream, p);
+  return hipGetLastError() == hipSuccess ? UA_OK : UA_ERR_LAUNCH;
+}

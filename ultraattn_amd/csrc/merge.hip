@@ -1,0 +1,171 @@
+// LSE-weighted merge of partial attention outputs, and the backward's row statistic
+// delta = rowsum(dO * O).  Both are HBM-bandwidth bound streaming kernels.
+//
+// A workgroup owns kTok consecutive tokens of all heads.  The per-row statistics are laid out
+// [batch, head, token] while the rows themselves are [batch, token, head, 128]; the workgroup
+// first handles the statistics with token-contiguous (coalesced) accesses and parks the row
+// weights in LDS, then streams the rows as 16-byte vectors (16 lanes per 256-byte row).
+#include "ua_common.h"
+
+namespace ua {
+
+constexpr int kTok = 16;          // tokens per workgroup
+constexpr int kMaxHeadsLds = 256; // rows per workgroup = kTok * n_heads <= 4096
+
+struct MergeParams {
+  const bf16* o_parts[UA_MAX_PARTS];
+  const float* lse_parts[UA_MAX_PARTS];
+  bf16* o; float* lse;
+  int n_parts, seqlen, n_heads;
+};
+
+template <int P>
+__global__ __launch_bounds__(256) void merge_kernel(const MergeParams p) {
+  extern __shared__ float w_lds[];              // [P][rows], rows = kTok * n_heads
+  const int tid = threadIdx.x;
+  const int tiles_per_batch = p.seqlen / kTok;
+  const int b = blockIdx.x / tiles_per_batch;
+  const int s0 = (blockIdx.x % tiles_per_batch) * kTok;
+  const int rows = kTok * p.n_heads;
+
+  // phase 1: one thread per (head, token): statistics, coalesced along the token axis
+  for (int t = tid; t < rows; t += 256) {
+    const int h = t / kTok, sl = t % kTok;
+    const int64_t li = ((int64_t)b * p.n_heads + h) * p.seqlen + s0 + sl;
+    float l[P];
+    float m = -INFINITY;
+#pragma unroll
+    for (int i = 0; i < P; ++i) { l[i] = p.lse_parts[i][li]; m = fmaxf(m, l[i]); }
+    const float ms = (m == -INFINITY) ? 0.f : m;
+    float den = 0.f;
+#pragma unroll
+    for (int i = 0; i < P; ++i) { l[i] = fast_exp2((l[i] - ms) * kLog2e); den += l[i]; }
+    const float inv = den > 0.f ? 1.f / den : 0.f;
+    const int row = sl * p.n_heads + h;
+#pragma unroll
+    for (int i = 0; i < P; ++i) w_lds[i * rows + row] = l[i] * inv;
+    p.lse[li] = den > 0.f ? ms + __builtin_amdgcn_logf(den) * kLn2 : -INFINITY;
+  }
+  __syncthreads();
+
+  // phase 2: stream the rows; chunk c covers 8 bf16 of row c/16
+  const int64_t base = ((int64_t)b * p.seqlen + s0) * p.n_heads * kHeadDim;
+  const int n_chunks = rows * 16;
+  for (int c = tid; c < n_chunks; c += 256) {
+    const int row = c >> 4;
+    u32x4 raw[P];
+#pragma unroll
+    for (int i = 0; i < P; ++i)
+      raw[i] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p.o_parts[i] + base) + c);
+    float acc[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) acc[j] = 0.f;
+#pragma unroll
+    for (int i = 0; i < P; ++i) {
+      const float w = w_lds[i * rows + row];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        acc[2 * j] = fmaf(w, __uint_as_float(raw[i][j] << 16), acc[2 * j]);
+        acc[2 * j + 1] = fmaf(w, __uint_as_float(raw[i][j] & 0xffff0000u), acc[2 * j + 1]);
+      }
+    }
+    bf16x8 out;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) out[j] = (bf16)acc[j];
+    __builtin_nontemporal_store(out, reinterpret_cast<bf16x8*>(p.o + base) + c);
+  }
+}
+
+struct DeltaParams {
+  const bf16* o; const bf16* dout; float* delta;
+  int seqlen, n_heads;
+  Strides3 os, ds;
+};
+
+__global__ __launch_bounds__(256) void delta_kernel(const DeltaParams p) {
+  extern __shared__ float d_lds[];               // [n_heads][kTok]
+  const int tid = threadIdx.x;
+  const int tiles_per_batch = p.seqlen / kTok;
+  const int b = blockIdx.x / tiles_per_batch;
+  const int s0 = (blockIdx.x % tiles_per_batch) * kTok;
+  const int rows = kTok * p.n_heads;
+  const int sub = tid & 15;
+  for (int row = tid >> 4; row < rows; row += 16) {
+    const int sl = row / p.n_heads, h = row % p.n_heads;
+    const int64_t s = s0 + sl;
+    const u32x4 a = *reinterpret_cast<const u32x4*>(p.o + b * p.os.b + s * p.os.s + h * p.os.h + sub * 8);
+    const u32x4 g = *reinterpret_cast<const u32x4*>(p.dout + b * p.ds.b + s * p.ds.s + h * p.ds.h + sub * 8);
+    float acc = 0.f;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      acc = fmaf(__uint_as_float(a[j] << 16), __uint_as_float(g[j] << 16), acc);
+      acc = fmaf(__uint_as_float(a[j] & 0xffff0000u), __uint_as_float(g[j] & 0xffff0000u), acc);
+    }
+    acc += __shfl_xor(acc, 1); acc += __shfl_xor(acc, 2); acc += __shfl_xor(acc, 4); acc += __shfl_xor(acc, 8);
+    if (sub == 0) d_lds[h * kTok + sl] = acc;
+  }
+  __syncthreads();
+  for (int t = tid; t < rows; t += 256) {
+    const int h = t / kTok, sl = t % kTok;
+    p.delta[((int64_t)b * p.n_heads + h) * p.seqlen + s0 + sl] = d_lds[t];
+  }
+}
+
+template <int P>
+static int launch_merge(const MergeParams& p, int blocks, size_t lds, hipStream_t st) {
+  hipLaunchKernelGGL(merge_kernel<P>, dim3(blocks), dim3(256), lds, st, p);
+  return hipGetLastError() == hipSuccess ? UA_OK : UA_ERR_LAUNCH;
+}
+
+}  // namespace ua
+
+extern "C" int ua_merge(const void* const* o_parts, const float* const* lse_parts, int n_parts,
+                        void* o, float* lse, int batch, int seqlen, int n_heads, int head_dim, void* stream) {
+  using namespace ua;
+  if (!o_parts || !lse_parts || !o || !lse) return UA_ERR_NULL;
+  if (n_parts < 1 || n_parts > UA_MAX_PARTS) return UA_ERR_UNSUPPORTED;
+  if (head_dim != kHeadDim) return UA_ERR_UNSUPPORTED;
+  if (batch <= 0 || seqlen <= 0 || n_heads <= 0 || seqlen % kTok != 0 || n_heads > kMaxHeadsLds) return UA_ERR_SHAPE;
+  if ((int64_t)batch * (seqlen / kTok) > INT32_MAX) return UA_ERR_SHAPE;
+  if (!aligned16(o)) return UA_ERR_ALIGN;
+  MergeParams p;
+  for (int i = 0; i < n_parts; ++i) {
+    if (!o_parts[i] || !lse_parts[i]) return UA_ERR_NULL;
+    if (!aligned16(o_parts[i])) return UA_ERR_ALIGN;
+    p.o_parts[i] = (const bf16*)o_parts[i];
+    p.lse_parts[i] = lse_parts[i];
+  }
+  for (int i = n_parts; i < UA_MAX_PARTS; ++i) { p.o_parts[i] = nullptr; p.lse_parts[i] = nullptr; }
+  p.o = (bf16*)o; p.lse = lse; p.n_parts = n_parts; p.seqlen = seqlen; p.n_heads = n_heads;
+  if (int rc = check_device()) return rc;
+  const int blocks = batch * (seqlen / kTok);
+  const size_t lds = (size_t)n_parts * kTok * n_heads * sizeof(float);
+  if (lds > 65536) return UA_ERR_SHAPE;   // n_parts * n_heads <= 1024
+  hipStream_t st = (hipStream_t)stream;
+  switch (n_parts) {
+#define UA_CASE(N) case N: return launch_merge<N>(p, blocks, lds, st);
+    UA_CASE(1) UA_CASE(2) UA_CASE(3) UA_CASE(4) UA_CASE(5) UA_CASE(6) UA_CASE(7) UA_CASE(8)
+    UA_CASE(9) UA_CASE(10) UA_CASE(11) UA_CASE(12) UA_CASE(13) UA_CASE(14) UA_CASE(15) UA_CASE(16)
+#undef UA_CASE
+  }
+  return UA_ERR_UNSUPPORTED;
+}
+
+extern "C" int ua_bsa_bwd_delta(const void* o, const void* dout, float* delta,
+                                int batch, int seqlen_q, int n_heads, int head_dim,
+                                const int64_t* o_strides, const int64_t* do_strides, void* stream) {
+  using namespace ua;
+  if (!o || !dout || !delta || !o_strides || !do_strides) return UA_ERR_NULL;
+  if (head_dim != kHeadDim) return UA_ERR_UNSUPPORTED;
+  if (batch <= 0 || seqlen_q <= 0 || n_heads <= 0 || seqlen_q % kTok != 0 || n_heads > kMaxHeadsLds) return UA_ERR_SHAPE;
+  if ((int64_t)batch * (seqlen_q / kTok) > INT32_MAX) return UA_ERR_SHAPE;
+  if (!aligned16(o) || !aligned16(dout) || !strides_ok(o_strides) || !strides_ok(do_strides)) return UA_ERR_ALIGN;
+  if (int rc = check_device()) return rc;
+  DeltaParams p;
+  p.o = (const bf16*)o; p.dout = (const bf16*)dout; p.delta = delta; p.seqlen = seqlen_q; p.n_heads = n_heads;
+  p.os = {o_strides[0], o_strides[1], o_strides[2]};
+  p.ds = {do_strides[0], do_strides[1], do_strides[2]};
+  hipLaunchKernelGGL(delta_kernel, dim3(batch * (seqlen_q / kTok)), dim3(256),
+                     (size_t)kTok * n_heads * sizeof(float), (hipStream_t)stream, p);
+  return hipGetLastError() == hipSuccess ? UA_OK : UA_ERR_LAUNCH;
+}

@@ -1,0 +1,179 @@
+// Block mask -> compacted active-tile list (CSR over query tiles, CSC over key tiles).
+//
+// Refinement rule (one block -> rate x rate tiles): EMPTY stays empty, FULL becomes all full,
+// CAUSAL becomes causal on the sub-diagonal, full below it and empty above it.  Tiles are
+// emitted row-major (query tile outer, key tile inner).
+#include <algorithm>
+#include <numeric>
+#include <vector>
+#include "ua_common.h"
+
+namespace ua {
+
+// type of tile (qt, kt): 0 empty, 1 full, 2 causal
+__host__ __device__ __forceinline__ int tile_type(const uint8_t* mask, int nkb, int rate, int qt, int kt) {
+  const int t = mask[(int64_t)(qt / rate) * nkb + kt / rate];
+  if (t != 2) return t;
+  const int a = qt % rate, b = kt % rate;
+  return a == b ? 2 : (a > b ? 1 : 0);
+}
+
+static int check_mask(const uint8_t* mask, int nqb, int nkb, int rate) {
+  if (!mask) return UA_ERR_NULL;
+  if (nqb <= 0 || nkb <= 0 || rate <= 0) return UA_ERR_SHAPE;
+  if ((int64_t)nqb * rate > (1 << 24) || (int64_t)nkb * rate > (1 << 24)) return UA_ERR_SHAPE;
+  for (int64_t i = 0; i < (int64_t)nqb * nkb; ++i)
+    if (mask[i] > 2) return UA_ERR_MASK;
+  return UA_OK;
+}
+
+// ---- device variant -----------------------------------------------------------------------
+// count: one thread per query tile (and per key tile) counts its active tiles.
+__global__ void tl_count_kernel(const uint8_t* mask, int nqb, int nkb, int rate, int32_t* qcnt, int32_t* kcnt) {
+  const int nqt = nqb * rate, nkt = nkb * rate;
+  const int t = blockIdx.x * blockDim.x + threadIdx.x;
+  if (t < nqt) {
+    int n = 0;
+    for (int kt = 0; kt < nkt; ++kt) n += tile_type(mask, nkb, rate, t, kt) != 0;
+    qcnt[t] = n;
+  } else if (t < nqt + nkt) {
+    const int kt = t - nqt;
+    int n = 0;
+    for (int q = 0; q < nqt; ++q) n += tile_type(mask, nkb, rate, q, kt) != 0;
+    kcnt[kt] = n;
+  }
+}
+
+// scan + order: a single workgroup turns counts into exclusive prefix sums and computes the
+// longest-first stable rank of every row by counting (rank = #rows that must come earlier).
+__global__ __launch_bounds__(1024) void tl_scan_kernel(const int32_t* cnt, int n, int32_t* ptr, int32_t* order) {
+  __shared__ int32_t part[1024];
+  const int tid = threadIdx.x;
+  const int per = (n + 1023) / 1024;
+  const int lo = min(n, tid * per), hi = min(n, lo + per);
+  int s = 0;
+  for (int i = lo; i < hi; ++i) s += cnt[i];
+  part[tid] = s;
+  __syncthreads();
+  for (int off = 1; off < 1024; off <<= 1) {
+    const int v = tid >= off ? part[tid - off] : 0;
+    __syncthreads();
+    part[tid] += v;
+    __syncthreads();
+  }
+  int run = tid ? part[tid - 1] : 0;
+  for (int i = lo; i < hi; ++i) { ptr[i] = run; run += cnt[i]; }
+  if (tid == 1023) ptr[n] = part[1023];
+  for (int i = tid; i < n; i += 1024) {
+    const int ci = cnt[i];
+    int rank = 0;
+    for (int j = 0; j < n; ++j) {
+      const int cj = cnt[j];
+      rank += (cj > ci) || (cj == ci && j < i);
+    }
+    order[rank] = i;
+  }
+}
+
+__global__ void tl_fill_kernel(const uint8_t* mask, int nqb, int nkb, int rate,
+                               const int32_t* row_ptr, int32_t* col_idx, uint8_t* flag,
+                               const int32_t* col_ptr, int32_t* row_idx, uint8_t* cflag) {
+  const int nqt = nqb * rate, nkt = nkb * rate;
+  const int t = blockIdx.x * blockDim.x + threadIdx.x;
+  if (t < nqt) {
+    int e = row_ptr[t];
+    for (int kt = 0; kt < nkt; ++kt) {
+      const int ty = tile_type(mask, nkb, rate, t, kt);
+      if (ty) { col_idx[e] = kt; flag[e] = ty == 2; ++e; }
+    }
+  } else if (t < nqt + nkt) {
+    const int kt = t - nqt;
+    int e = col_ptr[kt];
+    for (int q = 0; q < nqt; ++q) {
+      const int ty = tile_type(mask, nkb, rate, q, kt);
+      if (ty) { row_idx[e] = q; cflag[e] = ty == 2; ++e; }
+    }
+  }
+}
+
+}  // namespace ua
+
+extern "C" int ua_tilelist_size(const uint8_t* block_mask, int n_qblocks, int n_kblocks, int rate,
+                                int64_t* n_qtiles, int64_t* n_ktiles, int64_t* nnz) {
+  using namespace ua;
+  if (!n_qtiles || !n_ktiles || !nnz) return UA_ERR_NULL;
+  if (int rc = check_mask(block_mask, n_qblocks, n_kblocks, rate)) return rc;
+  int64_t n = 0;
+  for (int64_t i = 0; i < (int64_t)n_qblocks * n_kblocks; ++i) {
+    const int t = block_mask[i];
+    n += t == 1 ? (int64_t)rate * rate : (t == 2 ? (int64_t)rate * (rate + 1) / 2 : 0);
+  }
+  if (n > INT32_MAX) return UA_ERR_SHAPE;
+  *n_qtiles = (int64_t)n_qblocks * rate;
+  *n_ktiles = (int64_t)n_kblocks * rate;
+  *nnz = n;
+  return UA_OK;
+}
+
+extern "C" int ua_tilelist_build(const uint8_t* block_mask, int n_qblocks, int n_kblocks, int rate,
+                                 int32_t* row_ptr, int32_t* col_idx, uint8_t* flag,
+                                 int32_t* col_ptr, int32_t* row_idx, uint8_t* cflag,
+                                 int32_t* q_order, int32_t* k_order) {
+  using namespace ua;
+  if (int rc = check_mask(block_mask, n_qblocks, n_kblocks, rate)) return rc;
+  if (!row_ptr || !col_ptr || !q_order || !k_order) return UA_ERR_NULL;
+  const int nqt = n_qblocks * rate, nkt = n_kblocks * rate;
+  std::vector<int32_t> kcnt(nkt, 0);
+  int64_t e = 0;
+  for (int qt = 0; qt < nqt; ++qt) {
+    row_ptr[qt] = (int32_t)e;
+    for (int kb = 0; kb < n_kblocks; ++kb) {
+      if (!block_mask[(int64_t)(qt / rate) * n_kblocks + kb]) continue;
+      for (int kt = kb * rate; kt < (kb + 1) * rate; ++kt) {
+        const int ty = tile_type(block_mask, n_kblocks, rate, qt, kt);
+        if (!ty) continue;
+        if (!col_idx || !flag) return UA_ERR_NULL;
+        col_idx[e] = kt; flag[e] = ty == 2; ++e; ++kcnt[kt];
+      }
+    }
+  }
+  row_ptr[nqt] = (int32_t)e;
+  col_ptr[0] = 0;
+  for (int kt = 0; kt < nkt; ++kt) col_ptr[kt + 1] = col_ptr[kt] + kcnt[kt];
+  if (e > 0 && (!row_idx || !cflag)) return UA_ERR_NULL;
+  std::vector<int32_t> cur(col_ptr, col_ptr + nkt);
+  for (int qt = 0; qt < nqt; ++qt)
+    for (int32_t i = row_ptr[qt]; i < row_ptr[qt + 1]; ++i) {
+      const int32_t pos = cur[col_idx[i]]++;
+      row_idx[pos] = qt; cflag[pos] = flag[i];
+    }
+  std::iota(q_order, q_order + nqt, 0);
+  std::stable_sort(q_order, q_order + nqt, [&](int32_t a, int32_t b) {
+    return row_ptr[a + 1] - row_ptr[a] > row_ptr[b + 1] - row_ptr[b]; });
+  std::iota(k_order, k_order + nkt, 0);
+  std::stable_sort(k_order, k_order + nkt, [&](int32_t a, int32_t b) { return kcnt[a] > kcnt[b]; });
+  return UA_OK;
+}
+
+extern "C" int ua_tilelist_build_device(const uint8_t* block_mask, int n_qblocks, int n_kblocks, int rate,
+                                        int32_t* row_ptr, int32_t* col_idx, uint8_t* flag,
+                                        int32_t* col_ptr, int32_t* row_idx, uint8_t* cflag,
+                                        int32_t* q_order, int32_t* k_order, int32_t* work, void* stream) {
+  using namespace ua;
+  if (!block_mask || !row_ptr || !col_idx || !flag || !col_ptr || !row_idx || !cflag || !q_order || !k_order || !work)
+    return UA_ERR_NULL;
+  if (n_qblocks <= 0 || n_kblocks <= 0 || rate <= 0) return UA_ERR_SHAPE;
+  if ((int64_t)n_qblocks * rate > (1 << 24) || (int64_t)n_kblocks * rate > (1 << 24)) return UA_ERR_SHAPE;
+  if (int rc = check_device()) return rc;
+  const int nqt = n_qblocks * rate, nkt = n_kblocks * rate;
+  hipStream_t st = (hipStream_t)stream;
+  int32_t* qcnt = work;
+  int32_t* kcnt = work + nqt + 1;
+  const int blocks = (nqt + nkt + 255) / 256;
+  hipLaunchKernelGGL(tl_count_kernel, dim3(blocks), dim3(256), 0, st, block_mask, n_qblocks, n_kblocks, rate, qcnt, kcnt);
+  hipLaunchKernelGGL(tl_scan_kernel, dim3(1), dim3(1024), 0, st, (const int32_t*)qcnt, nqt, row_ptr, q_order);
+  hipLaunchKernelGGL(tl_scan_kernel, dim3(1), dim3(1024), 0, st, (const int32_t*)kcnt, nkt, col_ptr, k_order);
+  hipLaunchKernelGGL(tl_fill_kernel, dim3(blocks), dim3(256), 0, st, block_mask, n_qblocks, n_kblocks, rate,
+                     (const int32_t*)row_ptr, col_idx, flag, (const int32_t*)col_ptr, row_idx, cflag);
+  return hipGetLastError() == hipSuccess ? UA_OK : UA_ERR_LAUNCH;
+}
