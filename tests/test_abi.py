@@ -1,0 +1,78 @@
+"""The C-ABI library loads and exports every symbol that include/ultraattn.h declares; argument
+checks that need no GPU return the documented codes.  No GPU, no kernel launches."""
+import ctypes
+import os
+import re
+
+import numpy as np
+import pytest
+
+from ultraattn_amd import _lib
+from ultraattn_amd.build import LIB_PATH
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def declared_symbols():
+    text = open(os.path.join(ROOT, "include", "ultraattn.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(ua_[a-z_0-9]+)\s*\(", text)))
+
+
+def test_header_symbols_are_exported(lib):
+    names = declared_symbols()
+    assert {"ua_bsa_fwd", "ua_bsa_bwd_dkdv", "ua_bsa_bwd_dq", "ua_bsa_bwd_delta", "ua_merge",
+            "ua_tilelist_build", "ua_tilelist_size", "ua_tilelist_build_device", "ua_strerror",
+            "ua_version"} <= set(names)
+    raw = ctypes.CDLL(LIB_PATH)
+    for n in names:
+        assert hasattr(raw, n), f"{n} declared in include/ultraattn.h but not exported"
+    assert sorted(_lib.SIGNATURES) == names, "python binding and header disagree"
+    assert lib.ua_version() >= 100
+
+
+def test_argument_checks_without_gpu(lib):
+    s = (ctypes.c_int64 * 3)(128 * 128, 128, 128)
+    buf = np.zeros(64, np.uint8).ctypes.data // 16 * 16 + 16     # any aligned non-null address; never dereferenced
+    # NULL q
+    assert lib.ua_bsa_fwd(None, buf, buf, buf, buf, buf, buf, buf, buf, 1, 1, 1, 1, 128, s, s, s, s, 0.1, None) == -1
+    # head_dim != 128
+    assert lib.ua_bsa_fwd(buf, buf, buf, buf, buf, buf, buf, buf, buf, 1, 1, 1, 1, 64, s, s, s, s, 0.1, None) == -3
+    # non-positive scale
+    assert lib.ua_bsa_fwd(buf, buf, buf, buf, buf, buf, buf, buf, buf, 1, 1, 1, 1, 128, s, s, s, s, 0.0, None) == -3
+    # sizes
+    assert lib.ua_bsa_fwd(buf, buf, buf, buf, buf, buf, buf, buf, buf, 0, 1, 1, 1, 128, s, s, s, s, 0.1, None) == -2
+    # misaligned pointer / stride not a multiple of 8
+    assert lib.ua_bsa_fwd(buf + 2, buf, buf, buf, buf, buf, buf, buf, buf, 1, 1, 1, 1, 128, s, s, s, s, 0.1, None) == -4
+    bad = (ctypes.c_int64 * 3)(128 * 128, 132, 128)
+    assert lib.ua_bsa_fwd(buf, buf, buf, buf, buf, buf, buf, buf, buf, 1, 1, 1, 1, 128, bad, s, s, s, 0.1, None) == -4
+    # merge: too many partials, bad seqlen
+    arr = (ctypes.c_void_p * 17)(*([buf] * 17))
+    assert lib.ua_merge(arr, arr, 17, buf, buf, 1, 16, 1, 128, None) == -3
+    assert lib.ua_merge(arr, arr, 0, buf, buf, 1, 16, 1, 128, None) == -3
+    assert lib.ua_merge(arr, arr, 2, buf, buf, 1, 0, 1, 128, None) == -2
+    assert lib.ua_merge(None, arr, 2, buf, buf, 1, 16, 1, 128, None) == -1
+    # backward
+    assert lib.ua_bsa_bwd_delta(buf, None, buf, 1, 16, 1, 128, s, s, None) == -1
+    assert lib.ua_bsa_bwd_delta(buf, buf, buf, 1, 16, 1, 96, s, s, None) == -3
+    assert lib.ua_bsa_bwd_dq(buf, buf, buf, buf, buf, buf, None, buf, buf, buf, buf, 1, 1, 1, 1, 128,
+                             s, s, s, s, s, 0.1, None) in (-1, -7)
+    for code in range(-7, 1):
+        assert lib.ua_strerror(code) != b"unknown error code"
+    assert lib.ua_strerror(-99) == b"unknown error code"
+
+
+def test_missing_library_fails_loudly(monkeypatch, tmp_path):
+    monkeypatch.setattr(_lib, "_lib", None)
+    monkeypatch.setattr(_lib, "LIB_PATH", str(tmp_path / "nope.so"))
+    with pytest.raises(RuntimeError, match="no CPU or PyTorch fallback"):
+        _lib.load()
+
+
+def test_product_does_not_import_the_oracle():
+    pkg = os.path.join(ROOT, "ultraattn_amd")
+    for dirpath, _, files in os.walk(pkg):
+        for f in files:
+            if f.endswith(".py"):
+                src = open(os.path.join(dirpath, f)).read()
+                assert not re.search(r"^\s*(from|import)\s+oracle\b", src, flags=re.M), f

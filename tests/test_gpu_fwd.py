@@ -1,0 +1,159 @@
+"""Forward parity on the GPU, through the C ABI: HIP kernel vs the CPU oracle on the same
+seeded inputs, the committed golden twins, edge cases, and full-size sampled checks."""
+import math
+import os
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import attn_oracle as ao
+from tests.gpu_util import ATOL_O, RTOL_LSE, SCALE, lse_rel_err, max_abs, seeded_inputs, visible_keys_of_row
+from ultraattn_amd import masks, ops
+from ultraattn_amd.tilelist import build_tile_list
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+def run_fwd(q, k, v, mask, block, **kw):
+    o, lse = ops.bsa_fwd(q.to(DEV), k.to(DEV), v.to(DEV), mask, SCALE, block=block, **kw)
+    torch.cuda.synchronize()
+    return o, lse
+
+
+@pytest.mark.parametrize("name", ["c1_causal", "c3_strided", "c4_global_local", "c5_streaming"])
+def test_golden_twins(name, golden_dir):
+    from tests.golden.make_golden import twin_inputs
+    g = np.load(os.path.join(golden_dir, f"twin_{name}.npz"))
+    mask, block = g["mask"], int(g["block"])
+    q, k, v, _ = twin_inputs(mask, block, int(g["seed"]))
+    o, lse = run_fwd(q, k, v, mask, block)
+    assert max_abs(o[:, torch.from_numpy(g["qrows"]).to(DEV)], torch.from_numpy(g["o"])) <= ATOL_O
+    assert lse_rel_err(lse, torch.from_numpy(g["lse"])) <= RTOL_LSE
+
+
+CASES = {
+    "causal_4x4_b128": (lambda: masks.config_causal(4), 128, 2, 1),
+    "causal_2x2_b512": (lambda: masks.config_causal(2), 512, 2, 1),
+    "strided_16_b256": (lambda: masks.config_strided(16), 256, 8, 1),
+    "global_local_12": (lambda: masks.config_global_local(12, 1, 2), 128, 3, 1),
+    "stream_shard": (lambda: masks.config_streaming_shard(4, 16, 3), 128, 2, 1),
+    "batch2_heads5": (lambda: masks.config_causal(3), 128, 5, 2),
+    "single_full_tile": (lambda: np.ones((1, 1), np.uint8), 128, 1, 1),
+    "single_causal_tile": (lambda: np.full((1, 1), 2, np.uint8), 128, 1, 1),
+    "rect_1x6": (lambda: np.ones((1, 6), np.uint8), 128, 2, 1),
+    "canonical_stride": (lambda: masks.canonical_block_table(0), 128, 2, 1),
+    "canonical_stream": (lambda: masks.canonical_block_table(3), 256, 2, 1),
+}
+
+
+@pytest.mark.parametrize("case", list(CASES))
+@pytest.mark.parametrize("seed", [0, 1, 2])
+def test_fwd_vs_oracle(case, seed):
+    make, block, nh, batch = CASES[case]
+    mask = make()
+    q, k, v, _ = seeded_inputs(mask, block, seed, nh=nh, batch=batch)
+    o, lse = run_fwd(q, k, v, mask, block)
+    ro, rl = ao.dense_fwd(q, k, v, SCALE, ao.element_mask(mask, block))
+    assert max_abs(o, ro) <= ATOL_O
+    assert lse_rel_err(lse, rl) <= RTOL_LSE
+
+
+def test_rows_without_any_tile():
+    mask = np.zeros((3, 3), np.uint8)
+    mask[0, 0] = 2
+    mask[2, 1] = 1
+    q, k, v, _ = seeded_inputs(mask, 128, 0)
+    o, lse = run_fwd(q, k, v, mask, 128)
+    assert (o[:, 128:256] == 0).all()
+    assert torch.isinf(lse[:, :, 128:256]).all() and (lse[:, :, 128:256] < 0).all()
+    ro, rl = ao.dense_fwd(q, k, v, SCALE, ao.element_mask(mask, 128))
+    assert max_abs(o, ro) <= ATOL_O and lse_rel_err(lse, rl) <= RTOL_LSE
+    # an entirely empty mask
+    o, lse = run_fwd(q, k, v, np.zeros((3, 3), np.uint8), 128)
+    assert (o == 0).all() and torch.isinf(lse).all()
+
+
+def test_closed_forms_on_gpu():
+    mask = masks.config_causal(2)
+    q, k, v, _ = seeded_inputs(mask, 128, 3)
+    o, lse = run_fwd(torch.zeros_like(q), k, v, mask, 128)           # Q = 0: LSE = log(#visible keys)
+    want = torch.log(torch.arange(1, 257, dtype=torch.float32))
+    assert (lse.cpu() - want).abs().max() < 1e-4
+    vc = torch.full_like(v, 1.5)
+    o, _ = run_fwd(q, k, vc, mask, 128)                                  # constant V: O = constant
+    assert (o.float() - 1.5).abs().max() < 1e-2
+    o, lse = run_fwd(q, k, v, mask, 128)                                 # causal row 0: O = V[0]
+    assert torch.equal(o[0, 0].cpu(), v[0, 0])
+    assert (lse[0, :, 0].cpu() - SCALE * (q[0, 0].float() * k[0, 0].float()).sum(-1)).abs().max() < 1e-3
+
+
+def test_large_logits_stay_finite():
+    """Scores of magnitude ~60 (std-8 inputs): no overflow, LSE still within tolerance."""
+    mask = masks.config_causal(2)
+    q, k, v, _ = seeded_inputs(mask, 128, 5, std=8.0)
+    o, lse = run_fwd(q, k, v, mask, 128)
+    ro, rl = ao.dense_fwd(q, k, v, SCALE, ao.element_mask(mask, 128), dtype=torch.float64)
+    assert torch.isfinite(o).all()
+    assert lse_rel_err(lse, rl) <= RTOL_LSE
+    assert max_abs(o, ro) <= 8 * ATOL_O       # V has std 8: same relative bar
+
+
+def test_strided_views_and_out_argument():
+    """q/k/v/out as views into one packed buffer (the executor's Integrated_Data layout,
+    orchestrated_attn/utils.py:50-82) and in-place output."""
+    mask = masks.config_causal(2)
+    q, k, v, _ = seeded_inputs(mask, 128, 4, nh=4)
+    S, Nh, D = 256, 4, 128
+    packed = torch.zeros(1, S, 3 * Nh, D, dtype=torch.bfloat16, device=DEV)     # [q | k | v] along heads
+    packed[:, :, :Nh], packed[:, :, Nh:2 * Nh], packed[:, :, 2 * Nh:] = q.to(DEV), k.to(DEV), v.to(DEV)
+    out_buf = torch.full((1, S, 2 * Nh, D), 7.0, dtype=torch.bfloat16, device=DEV)
+    out = out_buf[:, :, Nh:]
+    o, lse = ops.bsa_fwd(packed[:, :, :Nh], packed[:, :, Nh:2 * Nh], packed[:, :, 2 * Nh:], mask, SCALE,
+                         block=128, out=out)
+    torch.cuda.synchronize()
+    assert o.data_ptr() == out.data_ptr()
+    assert (out_buf[:, :, :Nh] == 7.0).all()
+    ro, rl = ao.dense_fwd(q, k, v, SCALE, ao.element_mask(mask, 128))
+    assert max_abs(out, ro) <= ATOL_O and lse_rel_err(lse, rl) <= RTOL_LSE
+
+
+def test_argument_errors():
+    mask = masks.config_causal(2)
+    q, k, v, _ = seeded_inputs(mask, 128, 0)
+    qd, kd, vd = q.to(DEV), k.to(DEV), v.to(DEV)
+    with pytest.raises(TypeError):
+        ops.bsa_fwd(qd.float(), kd, vd, mask, SCALE)
+    with pytest.raises(ValueError):
+        ops.bsa_fwd(qd[:, :100], kd, vd, mask, SCALE)
+    with pytest.raises(ValueError):
+        ops.bsa_fwd(qd, kd, vd, masks.config_causal(3), SCALE, block=128)
+    with pytest.raises(ValueError):
+        ops.bsa_fwd(q, k, v, mask, SCALE)                  # CPU tensors: no CPU path
+    with pytest.raises(RuntimeError, match="unsupported"):
+        ops.bsa_fwd(qd, kd, vd, mask, -1.0)
+
+
+@pytest.mark.parametrize("cfg", ["c2", "c3", "c4", "c5"])
+def test_full_size_sampled_rows(cfg):
+    """The benchmark shapes (Nh = 32): sampled (row, head) pairs recomputed densely in fp32 with
+    the oracle's formula on the device, plus the size-independent bounds on LSE."""
+    mask = {"c2": masks.config_causal(64), "c3": masks.config_strided(), "c4": masks.config_global_local(),
+            "c5": masks.config_streaming_shard()}[cfg]
+    block, nh = 512, 32
+    g = torch.Generator(device=DEV).manual_seed(0)
+    mk = lambda n: torch.randn(1, n * block, nh, 128, device=DEV, dtype=torch.float32, generator=g).to(torch.bfloat16)
+    q, k, v = mk(mask.shape[0]), mk(mask.shape[1]), mk(mask.shape[1])
+    tl = build_tile_list(mask, block)
+    o, lse = ops.bsa_fwd(q, k, v, tl, SCALE)
+    torch.cuda.synchronize()
+    assert torch.isfinite(o).all() and torch.isfinite(lse).all()
+    rs = np.random.RandomState(0)
+    rows = list(rs.choice(q.shape[1], 24, replace=False)) + [0, 127, 128, 511, 512, q.shape[1] - 1]
+    for row in rows:
+        h = int(rs.randint(nh))
+        vis = visible_keys_of_row(mask, block, int(row)).to(DEV)
+        ro, rl = ao.dense_fwd(q[:, row:row + 1, h:h + 1], k[:, :, h:h + 1], v[:, :, h:h + 1], SCALE, vis[None, :])
+        assert (o[0, row, h].float() - ro[0, 0, 0]).abs().max().item() <= ATOL_O, (row, h)
+        assert abs(lse[0, h, row].item() - rl.item()) <= RTOL_LSE * max(1.0, abs(rl.item())), (row, h)

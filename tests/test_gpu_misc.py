@@ -1,0 +1,71 @@
+"""Device-side tile-list builder (bit-exact) and the flash-attn call-signature shim, on the GPU."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import attn_oracle as ao
+from oracle import tilelist_oracle as to
+from tests.gpu_util import ATOL_O, RTOL_LSE, SCALE, lse_rel_err, max_abs, seeded_inputs
+from ultraattn_amd import masks
+from ultraattn_amd.flash_attn_interface import _flash_attn_backward, _flash_attn_forward
+from ultraattn_amd.tilelist import build_tile_list, build_tile_list_device
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+FIELDS = ("row_ptr", "col_idx", "flag", "col_ptr", "row_idx", "cflag", "q_order", "k_order")
+
+
+@pytest.mark.parametrize("make,block", [
+    (lambda: masks.config_causal(16), 512), (lambda: masks.config_strided(), 512),
+    (lambda: masks.config_global_local(), 512), (lambda: masks.config_streaming_shard(), 512),
+    (lambda: masks.canonical_block_table(3), 1024), (lambda: np.zeros((2, 3), np.uint8), 256),
+    (lambda: np.random.RandomState(3).randint(0, 3, size=(7, 5)).astype(np.uint8), 384),
+])
+def test_device_builder_bit_exact(make, block):
+    m = make()
+    host = build_tile_list(m, block)
+    oracle = to.build_tile_list(m, block // 128)
+    dev = build_tile_list_device(torch.from_numpy(m).to(DEV), block, nnz=host.nnz)
+    torch.cuda.synchronize()
+    for f in FIELDS:
+        got = dev[f].cpu().numpy()
+        assert got.dtype == oracle[f].dtype and np.array_equal(got, oracle[f]), f
+        assert np.array_equal(got, getattr(host, f)), f
+
+
+@pytest.mark.parametrize("causal", [False, True])
+@pytest.mark.parametrize("sq,sk", [(256, 256), (128, 384), (384, 384)])
+def test_flash_attn_shim(causal, sq, sk):
+    """Same call as fwd_comp_func / bwd_comp_func make (orchestrated_attn_impl.py:326-337,
+    578-596), checked against the oracle's dense tile."""
+    if causal and sq != sk:
+        pytest.skip("the reference only runs causal tiles on square diagonal chunks")
+    g = torch.Generator().manual_seed(sq + sk)
+    mk = lambda n: torch.randn(1, n, 3, 128, generator=g).to(torch.bfloat16)
+    q, k, v, do = mk(sq), mk(sk), mk(sk), mk(sq)
+    qd, kd, vd, dod = (t.to(DEV) for t in (q, k, v, do))
+    out_buf = torch.empty_like(qd)
+    res = _flash_attn_forward(qd, kd, vd, 0.0, SCALE, causal=causal, window_size=(-1, -1), alibi_slopes=None,
+                              return_softmax=False, out=out_buf)
+    assert len(res) == 8 and res[0].data_ptr() == out_buf.data_ptr()
+    O, lse = res[0], res[5]
+    ro, rl = ao.tile_fwd(q, k, v, SCALE, causal)
+    assert lse.shape == (1, 3, sq)
+    assert max_abs(O, ro) <= ATOL_O and lse_rel_err(lse, rl) <= RTOL_LSE
+    delta = ao.softmax_delta(ro, do).to(DEV)
+    dq, dk, dv = torch.empty_like(qd), torch.empty_like(kd), torch.empty_like(vd)
+    _flash_attn_backward(dod, qd, kd, vd, qd, lse, dq, dk, dv, 0.0, SCALE, causal, (-1, -1), None, False,
+                         rng_state=None, softmax_d=delta)
+    torch.cuda.synchronize()
+    rq, rk, rv = ao.tile_bwd(do, q, k, v, rl, ao.softmax_delta(ro, do), SCALE, causal)
+    assert max_abs(dq, rq) <= ATOL_O and max_abs(dk, rk) <= ATOL_O and max_abs(dv, rv) <= ATOL_O
+
+
+def test_shim_rejects_unsupported_features():
+    q = torch.zeros(1, 128, 1, 128, dtype=torch.bfloat16, device=DEV)
+    with pytest.raises(NotImplementedError):
+        _flash_attn_forward(q, q, q, 0.1, SCALE, causal=False)
+    with pytest.raises(NotImplementedError):
+        _flash_attn_forward(q, q, q, 0.0, SCALE, causal=False, window_size=(64, 0))
+    with pytest.raises(NotImplementedError):
+        _flash_attn_forward(q, q, q, 0.0, SCALE, causal=False, alibi_slopes=torch.ones(1))

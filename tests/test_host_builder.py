@@ -1,0 +1,91 @@
+"""The C-ABI tile-list builder (host entry points) against the numpy oracle: bit-exact.  No GPU."""
+import ctypes
+import json
+import os
+
+import numpy as np
+import pytest
+from hypothesis import given, settings
+from hypothesis import strategies as st
+
+from oracle import tilelist_oracle as to
+from ultraattn_amd import _lib, masks
+from ultraattn_amd.tilelist import build_tile_list
+
+FIELDS = ("row_ptr", "col_idx", "flag", "col_ptr", "row_idx", "cflag", "q_order", "k_order")
+
+
+def assert_same(tl, ref):
+    assert tl.n_qtiles == ref["n_qtiles"] and tl.n_ktiles == ref["n_ktiles"]
+    for f in FIELDS:
+        a, b = getattr(tl, f), ref[f]
+        assert a.dtype == b.dtype and np.array_equal(a, b), f
+
+
+@pytest.mark.parametrize("make,rate", [
+    (lambda: masks.config_causal(16), 4), (lambda: masks.config_strided(48), 4),
+    (lambda: masks.config_global_local(40), 2), (lambda: masks.config_streaming_shard(8, 64, 5), 4),
+    (lambda: masks.canonical_block_table(0), 1), (lambda: masks.canonical_block_table(3), 8),
+    (lambda: np.zeros((3, 4), np.uint8), 2), (lambda: np.full((1, 1), 2, np.uint8), 5),
+])
+def test_builder_bit_exact(make, rate, lib):
+    m = make()
+    assert_same(build_tile_list(m, block=128 * rate), to.build_tile_list(m, rate))
+
+
+@settings(max_examples=60, deadline=None)
+@given(st.integers(1, 9), st.integers(1, 9), st.integers(1, 4), st.integers(0, 2 ** 31 - 1))
+def test_builder_bit_exact_random(nq, nk, rate, seed):
+    m = np.random.RandomState(seed).randint(0, 3, size=(nq, nk)).astype(np.uint8)
+    assert_same(build_tile_list(m, block=128 * rate), to.build_tile_list(m, rate))
+
+
+def test_full_size_digests(golden_dir, lib):
+    gold = json.load(open(os.path.join(golden_dir, "tilelists.json")))
+    cfgs = {"c1": masks.config_causal(16), "c2": masks.config_causal(64), "c3": masks.config_strided(),
+            "c4": masks.config_global_local(), "c5": masks.config_streaming_shard()}
+    for k, m in cfgs.items():
+        tl = build_tile_list(m, block=512)
+        assert tl.nnz == gold[k]["tiles"] and tl.n_causal == gold[k]["causal_tiles"]
+        assert tl.sha256() == gold[k]["sha256"]
+        # CSC is the transpose of the CSR
+        pairs = sorted((int(c), r) for r in range(tl.n_qtiles) for c in tl.col_idx[tl.row_ptr[r]:tl.row_ptr[r + 1]])
+        csc = [(c, int(r)) for c in range(tl.n_ktiles) for r in tl.row_idx[tl.col_ptr[c]:tl.col_ptr[c + 1]]]
+        assert pairs == csc
+        # orders are permutations sorted by length, longest first, ties by index
+        ql = np.diff(tl.row_ptr)
+        assert sorted(tl.q_order.tolist()) == list(range(tl.n_qtiles))
+        assert all((ql[a], -a) >= (ql[b], -b) for a, b in zip(tl.q_order[:-1], tl.q_order[1:]))
+
+
+def test_causal_flag_and_offset(lib):
+    ones = np.ones((2, 4), np.uint8)
+    tl = build_tile_list(ones, block=256, causal=True, q_block_offset=2)
+    ref = to.build_tile_list(to.apply_causal_rule(ones, True, 2), 2)
+    assert_same(tl, ref)
+    assert tl.n_causal == 4
+    tl0 = build_tile_list(ones, block=256, causal=False)
+    assert tl0.n_causal == 0 and tl0.nnz == 32
+    boolean = build_tile_list(np.ones((2, 2), bool), block=128, causal=True)
+    assert boolean.flag.tolist() == [1, 1, 1, 0] or boolean.n_causal == 2
+
+
+def test_error_codes(lib):
+    m = np.array([[1, 3]], np.uint8)
+    n = (ctypes.c_int64 * 3)()
+    p = lambda i: ctypes.byref(n, 8 * i)
+    sz = lambda mask, a, b, r: lib.ua_tilelist_size(mask, a, b, r, ctypes.cast(p(0), _lib._i64p),
+                                                     ctypes.cast(p(1), _lib._i64p), ctypes.cast(p(2), _lib._i64p))
+    assert sz(m.ctypes.data, 1, 2, 1) == -5                     # UA_ERR_MASK
+    assert sz(None, 1, 2, 1) == -1                               # UA_ERR_NULL
+    ok = np.ones((1, 2), np.uint8)
+    assert sz(ok.ctypes.data, 0, 2, 1) == -2                     # UA_ERR_SHAPE
+    assert sz(ok.ctypes.data, 1, 2, 0) == -2
+    assert sz(ok.ctypes.data, 1, 2, 3) == 0 and list(n) == [3, 6, 18]
+    assert b"EMPTY" in lib.ua_strerror(-5) and lib.ua_strerror(0) == b"ok"
+    with pytest.raises(RuntimeError, match="mask"):
+        build_tile_list(m, block=128)
+    with pytest.raises(ValueError):
+        build_tile_list(ok, block=100)
+    with pytest.raises(ValueError):
+        build_tile_list(np.ones(3, np.uint8), block=128)

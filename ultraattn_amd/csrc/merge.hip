@@ -23,14 +23,16 @@ template <int P>
 __global__ __launch_bounds__(256) void merge_kernel(const MergeParams p) {
   extern __shared__ float w_lds[];              // [P][rows], rows = kTok * n_heads
   const int tid = threadIdx.x;
-  const int tiles_per_batch = p.seqlen / kTok;
+  const int tiles_per_batch = (p.seqlen + kTok - 1) / kTok;
   const int b = blockIdx.x / tiles_per_batch;
   const int s0 = (blockIdx.x % tiles_per_batch) * kTok;
-  const int rows = kTok * p.n_heads;
+  const int ntok = min(kTok, p.seqlen - s0);       // the last workgroup of a batch may be ragged
+  const int rows = ntok * p.n_heads;
 
   // phase 1: one thread per (head, token): statistics, coalesced along the token axis
-  for (int t = tid; t < rows; t += 256) {
+  for (int t = tid; t < kTok * p.n_heads; t += 256) {
     const int h = t / kTok, sl = t % kTok;
+    if (sl >= ntok) continue;
     const int64_t li = ((int64_t)b * p.n_heads + h) * p.seqlen + s0 + sl;
     float l[P];
     float m = -INFINITY;
@@ -85,10 +87,11 @@ struct DeltaParams {
 __global__ __launch_bounds__(256) void delta_kernel(const DeltaParams p) {
   extern __shared__ float d_lds[];               // [n_heads][kTok]
   const int tid = threadIdx.x;
-  const int tiles_per_batch = p.seqlen / kTok;
+  const int tiles_per_batch = (p.seqlen + kTok - 1) / kTok;
   const int b = blockIdx.x / tiles_per_batch;
   const int s0 = (blockIdx.x % tiles_per_batch) * kTok;
-  const int rows = kTok * p.n_heads;
+  const int ntok = min(kTok, p.seqlen - s0);
+  const int rows = ntok * p.n_heads;
   const int sub = tid & 15;
   for (int row = tid >> 4; row < rows; row += 16) {
     const int sl = row / p.n_heads, h = row % p.n_heads;
@@ -105,8 +108,9 @@ __global__ __launch_bounds__(256) void delta_kernel(const DeltaParams p) {
     if (sub == 0) d_lds[h * kTok + sl] = acc;
   }
   __syncthreads();
-  for (int t = tid; t < rows; t += 256) {
+  for (int t = tid; t < kTok * p.n_heads; t += 256) {
     const int h = t / kTok, sl = t % kTok;
+    if (sl >= ntok) continue;
     p.delta[((int64_t)b * p.n_heads + h) * p.seqlen + s0 + sl] = d_lds[t];
   }
 }
@@ -125,8 +129,8 @@ extern "C" int ua_merge(const void* const* o_parts, const float* const* lse_part
   if (!o_parts || !lse_parts || !o || !lse) return UA_ERR_NULL;
   if (n_parts < 1 || n_parts > UA_MAX_PARTS) return UA_ERR_UNSUPPORTED;
   if (head_dim != kHeadDim) return UA_ERR_UNSUPPORTED;
-  if (batch <= 0 || seqlen <= 0 || n_heads <= 0 || seqlen % kTok != 0 || n_heads > kMaxHeadsLds) return UA_ERR_SHAPE;
-  if ((int64_t)batch * (seqlen / kTok) > INT32_MAX) return UA_ERR_SHAPE;
+  if (batch <= 0 || seqlen <= 0 || n_heads <= 0 || n_heads > kMaxHeadsLds) return UA_ERR_SHAPE;
+  if ((int64_t)batch * ((seqlen + kTok - 1) / kTok) > INT32_MAX) return UA_ERR_SHAPE;
   if (!aligned16(o)) return UA_ERR_ALIGN;
   MergeParams p;
   for (int i = 0; i < n_parts; ++i) {
@@ -138,7 +142,7 @@ extern "C" int ua_merge(const void* const* o_parts, const float* const* lse_part
   for (int i = n_parts; i < UA_MAX_PARTS; ++i) { p.o_parts[i] = nullptr; p.lse_parts[i] = nullptr; }
   p.o = (bf16*)o; p.lse = lse; p.n_parts = n_parts; p.seqlen = seqlen; p.n_heads = n_heads;
   if (int rc = check_device()) return rc;
-  const int blocks = batch * (seqlen / kTok);
+  const int blocks = batch * ((seqlen + kTok - 1) / kTok);
   const size_t lds = (size_t)n_parts * kTok * n_heads * sizeof(float);
   if (lds > 65536) return UA_ERR_SHAPE;   // n_parts * n_heads <= 1024
   hipStream_t st = (hipStream_t)stream;
@@ -157,15 +161,15 @@ extern "C" int ua_bsa_bwd_delta(const void* o, const void* dout, float* delta,
   using namespace ua;
   if (!o || !dout || !delta || !o_strides || !do_strides) return UA_ERR_NULL;
   if (head_dim != kHeadDim) return UA_ERR_UNSUPPORTED;
-  if (batch <= 0 || seqlen_q <= 0 || n_heads <= 0 || seqlen_q % kTok != 0 || n_heads > kMaxHeadsLds) return UA_ERR_SHAPE;
-  if ((int64_t)batch * (seqlen_q / kTok) > INT32_MAX) return UA_ERR_SHAPE;
+  if (batch <= 0 || seqlen_q <= 0 || n_heads <= 0 || n_heads > kMaxHeadsLds) return UA_ERR_SHAPE;
+  if ((int64_t)batch * ((seqlen_q + kTok - 1) / kTok) > INT32_MAX) return UA_ERR_SHAPE;
   if (!aligned16(o) || !aligned16(dout) || !strides_ok(o_strides) || !strides_ok(do_strides)) return UA_ERR_ALIGN;
   if (int rc = check_device()) return rc;
   DeltaParams p;
   p.o = (const bf16*)o; p.dout = (const bf16*)dout; p.delta = delta; p.seqlen = seqlen_q; p.n_heads = n_heads;
   p.os = {o_strides[0], o_strides[1], o_strides[2]};
   p.ds = {do_strides[0], do_strides[1], do_strides[2]};
-  hipLaunchKernelGGL(delta_kernel, dim3(batch * (seqlen_q / kTok)), dim3(256),
+  hipLaunchKernelGGL(delta_kernel, dim3(batch * ((seqlen_q + kTok - 1) / kTok)), dim3(256),
                      (size_t)kTok * n_heads * sizeof(float), (hipStream_t)stream, p);
   return hipGetLastError() == hipSuccess ? UA_OK : UA_ERR_LAUNCH;
 }

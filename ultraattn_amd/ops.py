@@ -17,7 +17,7 @@ from .tilelist import TILE, TileList, build_tile_list
 HEAD_DIM = 128
 
 
-def _check_qkv(name: str, t: torch.Tensor) -> None:
+def _check_qkv(name: str, t: torch.Tensor, seq_multiple: int = TILE) -> None:
     if not t.is_cuda:
         raise ValueError(f"{name} must be a CUDA (HIP) tensor")
     if t.dtype != torch.bfloat16:
@@ -26,8 +26,8 @@ def _check_qkv(name: str, t: torch.Tensor) -> None:
         raise ValueError(f"{name} must be [B, S, Nh, {HEAD_DIM}], got {tuple(t.shape)}")
     if t.stride(-1) != 1:
         raise ValueError(f"{name}: head_dim axis must be contiguous")
-    if t.shape[1] % TILE != 0:
-        raise ValueError(f"{name}: sequence length {t.shape[1]} is not a multiple of {TILE}")
+    if t.shape[1] % seq_multiple != 0:
+        raise ValueError(f"{name}: sequence length {t.shape[1]} is not a multiple of {seq_multiple}")
 
 
 def _tiles_for(tiles: Union[TileList, np.ndarray, torch.Tensor], q, k, block, causal, q_block_offset) -> TileList:
@@ -91,8 +91,10 @@ def bsa_fwd(q, k, v, tiles, softmax_scale: Optional[float] = None, causal: bool 
 def softmax_delta(out, dout, delta: Optional[torch.Tensor] = None) -> torch.Tensor:
     """delta = rowsum(dout * out) as fp32 [B, Nh, Sq]: the ``softmax_d`` input of the fork's
     backward (``orchestrated_attn/orchestrated_attn_impl.py:595``)."""
-    _check_qkv("out", out)
-    _check_qkv("dout", dout)
+    _check_qkv("out", out, 1)
+    _check_qkv("dout", dout, 1)
+    if out.shape != dout.shape:
+        raise ValueError("out and dout must have the same shape")
     B, Sq, Nh, D = out.shape
     if delta is None:
         delta = torch.empty(B, Nh, Sq, dtype=torch.float32, device=out.device)
@@ -164,7 +166,7 @@ def merge_partials(outs: Sequence[torch.Tensor], lses: Sequence[torch.Tensor],
         raise ValueError("need as many lses as outs, at least one")
     B, S, Nh, D = outs[0].shape
     for o_, l_ in zip(outs, lses):
-        _check_qkv("partial out", o_)
+        _check_qkv("partial out", o_, 1)
         if o_.shape != outs[0].shape or not o_.is_contiguous():
             raise ValueError("partial outs must be contiguous and of equal shape")
         if l_.shape != (B, Nh, S) or l_.dtype != torch.float32 or not l_.is_contiguous():

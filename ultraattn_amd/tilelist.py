@@ -104,11 +104,12 @@ def build_tile_list_device(block_mask_dev, block: int = 512, nnz: Optional[int] 
     nqb, nkb = m.shape
     nqt, nkt = nqb * rate, nkb * rate
     cap = nnz if nnz is not None else nqt * nkt
+    alloc = max(cap, 1)          # keep the pointers non-NULL for an empty list
     dev = m.device
     i32 = dict(dtype=torch.int32, device=dev)
     u8 = dict(dtype=torch.uint8, device=dev)
-    out = dict(row_ptr=torch.empty(nqt + 1, **i32), col_idx=torch.empty(cap, **i32), flag=torch.empty(cap, **u8),
-               col_ptr=torch.empty(nkt + 1, **i32), row_idx=torch.empty(cap, **i32), cflag=torch.empty(cap, **u8),
+    out = dict(row_ptr=torch.empty(nqt + 1, **i32), col_idx=torch.empty(alloc, **i32), flag=torch.empty(alloc, **u8),
+               col_ptr=torch.empty(nkt + 1, **i32), row_idx=torch.empty(alloc, **i32), cflag=torch.empty(alloc, **u8),
                q_order=torch.empty(nqt, **i32), k_order=torch.empty(nkt, **i32))
     work = torch.empty(nqt + nkt + 2, **i32)
     lib = _lib.load()
@@ -117,4 +118,6 @@ def build_tile_list_device(block_mask_dev, block: int = 512, nnz: Optional[int] 
         _lib.check(lib.ua_tilelist_build_device(m.data_ptr(), nqb, nkb, rate,
                                                 *[out[n].data_ptr() for n in _HOST_FIELDS],
                                                 work.data_ptr(), st), "ua_tilelist_build_device")
+    for n in ("col_idx", "flag", "row_idx", "cflag"):
+        out[n] = out[n][:cap]
     return out
