@@ -1,0 +1,314 @@
+#!/usr/bin/env python3
+"""Benchmark of the block-sparse attention hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c3|c4|c2|c5] [--no-extra] [--no-cpu]
+
+A step is one pass of the hot path over one batch of synthetic input: forward, delta, dK/dV and
+dQ for the forward+backward workloads (c3 = strided 128k, the default; c4 = global+local 128k),
+forward only for c2 (causal 32k) and forward tiles + merge for c5 (streaming shard).  Inputs are
+resident in HBM before the timed region.  Prints ONE JSON line on stdout; progress goes to stderr.
+"""
+import argparse
+import json
+import math
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+BLOCK = 512
+HEADS = 32
+SCALE = 1.0 / math.sqrt(128)
+HBM_PEAK_GBPS = 8000.0            # MI355X HBM3E, published
+FLOP_PER_CLK_PER_CU = 4096        # dense bf16 MFMA, CDNA4
+
+
+def log(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+def workload_mask(name):
+    from ultraattn_amd import masks
+    return {"c2": masks.config_causal(64), "c3": masks.config_strided(), "c4": masks.config_global_local(),
+            "c5": masks.config_streaming_shard()}[name]
+
+
+def fwd_flops(mask, nh=HEADS, block=BLOCK):
+    """Reference convention (search_algo/utils.py:92-103): 4*Sq*Skv*Nh*D*density, CAUSAL = 0.5."""
+    nf, nc = int((mask == 1).sum()), int((mask == 2).sum())
+    return 4.0 * block * block * 128 * nh * (nf + 0.5 * nc)
+
+
+class Timer:
+    """HIP events on the stream the kernels are launched on (torch's current stream)."""
+
+    def __init__(self, torch, names):
+        self.torch, self.names = torch, names
+        self.acc = {n: 0.0 for n in names}
+        self.marks = []
+
+    def mark(self):
+        e = self.torch.cuda.Event(enable_timing=True)
+        e.record()
+        self.marks.append(e)
+
+    def collect(self):
+        """Call after a synchronize: fold the recorded marks into per-kernel sums."""
+        per = len(self.names) + 1
+        for i in range(0, len(self.marks), per):
+            for j, n in enumerate(self.names):
+                self.acc[n] += self.marks[i + j].elapsed_time(self.marks[i + j + 1])
+        self.marks = []
+
+
+def run_attention(name, steps, warmup, backward):
+    import torch
+    from ultraattn_amd import ops
+    from ultraattn_amd.tilelist import build_tile_list
+    dev = "cuda:0"
+    mask = workload_mask(name)
+    nqb, nkb = mask.shape
+    g = torch.Generator(device=dev).manual_seed(0)
+    mk = lambda n: torch.randn(1, n * BLOCK, HEADS, 128, device=dev, dtype=torch.float32, generator=g).to(torch.bfloat16)
+    q, k, v = mk(nqb), mk(nkb), mk(nkb)
+    t0 = time.perf_counter()
+    tl = build_tile_list(mask, BLOCK)
+    tl.on(dev)
+    t_build = time.perf_counter() - t0
+    o = torch.empty_like(q)
+    lse = torch.empty(1, HEADS, nqb * BLOCK, dtype=torch.float32, device=dev)
+    names = ["fwd"]
+    if backward:
+        do = mk(nqb)
+        dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+        delta = torch.empty_like(lse)
+        names += ["delta", "bwd"]
+
+    def step(t=None):
+        if t: t.mark()
+        ops.bsa_fwd(q, k, v, tl, SCALE, out=o, lse=lse)
+        if t: t.mark()
+        if backward:
+            ops.softmax_delta(o, do, delta)
+            if t: t.mark()
+            ops.bsa_bwd(do, q, k, v, None, lse, tl, SCALE, dq=dq, dk=dk, dv=dv, softmax_d=delta)
+            if t: t.mark()
+
+    for _ in range(warmup):
+        step()
+    torch.cuda.synchronize()
+    timer = Timer(torch, names)
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        step(timer)
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3 / steps
+    timer.collect()
+    F = fwd_flops(mask)
+    ms = {n: timer.acc[n] / steps for n in names}
+    res = {"workload": name, "tiles_per_head": tl.nnz, "tilelist_sha256": tl.sha256(), "tilelist_build_ms": t_build * 1e3,
+           "ms_per_step": wall_ms, "fwd_ms": ms["fwd"], "fwd_tflops": F / ms["fwd"] / 1e9, "fwd_flops": F}
+    if backward:
+        res.update(bwd_ms=ms["bwd"], delta_ms=ms["delta"], bwd_tflops=2.5 * F / (ms["bwd"] + ms["delta"]) / 1e9,
+                   fwd_bwd_tflops=3.5 * F / wall_ms / 1e9,
+                   delta_gbps=(2 * q.numel() * 2 + lse.numel() * 4) / ms["delta"] / 1e6)
+    return res
+
+
+def time_bwd_kernels(name, steps):
+    """Separate event timing of the two backward kernels (dK/dV walks the CSC, dQ the CSR)."""
+    import ctypes
+    import torch
+    from ultraattn_amd import _lib, ops
+    from ultraattn_amd.tilelist import build_tile_list
+    dev = "cuda:0"
+    mask = workload_mask(name)
+    g = torch.Generator(device=dev).manual_seed(0)
+    mk = lambda n: torch.randn(1, n * BLOCK, HEADS, 128, device=dev, dtype=torch.float32, generator=g).to(torch.bfloat16)
+    q, k, v, do = mk(mask.shape[0]), mk(mask.shape[1]), mk(mask.shape[1]), mk(mask.shape[0])
+    tl = build_tile_list(mask, BLOCK)
+    d = tl.on(dev)
+    o, lse = ops.bsa_fwd(q, k, v, tl, SCALE)
+    delta = ops.softmax_delta(o, do)
+    dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+    lib = _lib.load()
+    st = torch.cuda.current_stream().cuda_stream
+    s3 = _lib.strides3
+
+    def dkdv():
+        _lib.check(lib.ua_bsa_bwd_dkdv(q.data_ptr(), k.data_ptr(), v.data_ptr(), do.data_ptr(), lse.data_ptr(),
+                                       delta.data_ptr(), dk.data_ptr(), dv.data_ptr(), d["col_ptr"].data_ptr(),
+                                       d["row_idx"].data_ptr(), d["cflag"].data_ptr(), d["k_order"].data_ptr(),
+                                       1, HEADS, tl.n_qtiles, tl.n_ktiles, 128, s3(q), s3(k), s3(v), s3(do), s3(dk),
+                                       s3(dv), SCALE, st), "dkdv")
+
+    def dqk():
+        _lib.check(lib.ua_bsa_bwd_dq(q.data_ptr(), k.data_ptr(), v.data_ptr(), do.data_ptr(), lse.data_ptr(),
+                                     delta.data_ptr(), dq.data_ptr(), d["row_ptr"].data_ptr(), d["col_idx"].data_ptr(),
+                                     d["flag"].data_ptr(), d["q_order"].data_ptr(), 1, HEADS, tl.n_qtiles,
+                                     tl.n_ktiles, 128, s3(q), s3(k), s3(v), s3(do), s3(dq), SCALE, st), "dq")
+    dkdv(); dqk()
+    torch.cuda.synchronize()
+    t = Timer(torch, ["dkdv", "dq"])
+    for _ in range(steps):
+        t.mark(); dkdv(); t.mark(); dqk(); t.mark()
+    torch.cuda.synchronize()
+    t.collect()
+    return {n: t.acc[n] / steps for n in t.names}
+
+
+def run_c5(steps, warmup):
+    """Streaming shard: 4 key-range kernel tiles -> partial (O, LSE) -> merge."""
+    import numpy as np
+    import torch
+    from ultraattn_amd import ops
+    from ultraattn_amd.tilelist import build_tile_list
+    dev = "cuda:0"
+    mask = workload_mask("c5")
+    nqb, nkb = mask.shape
+    g = torch.Generator(device=dev).manual_seed(0)
+    mk = lambda n: torch.randn(1, n * BLOCK, HEADS, 128, device=dev, dtype=torch.float32, generator=g).to(torch.bfloat16)
+    q, k, v = mk(nqb), mk(nkb), mk(nkb)
+    cols = np.nonzero(mask.any(0))[0]
+    tls = []
+    for c in np.array_split(cols, 4):
+        sub = np.zeros_like(mask)
+        sub[:, c] = mask[:, c]
+        tls.append(build_tile_list(sub, BLOCK))
+    p_o = [torch.empty_like(q) for _ in tls]
+    p_l = [torch.empty(1, HEADS, nqb * BLOCK, dtype=torch.float32, device=dev) for _ in tls]
+    o, lse = torch.empty_like(q), torch.empty_like(p_l[0])
+
+    def step(t=None):
+        if t: t.mark()
+        for tl, po, pl in zip(tls, p_o, p_l):
+            ops.bsa_fwd(q, k, v, tl, SCALE, out=po, lse=pl)
+        if t: t.mark()
+        ops.merge_partials(p_o, p_l, out=o, lse=lse)
+        if t: t.mark()
+
+    for _ in range(warmup):
+        step()
+    torch.cuda.synchronize()
+    timer = Timer(torch, ["fwd_tiles", "merge"])
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        step(timer)
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3 / steps
+    timer.collect()
+    F = fwd_flops(mask)
+    rows = nqb * BLOCK * HEADS
+    merge_bytes = (len(tls) + 1) * rows * (128 * 2 + 4)
+    m_ms, f_ms = timer.acc["merge"] / steps, timer.acc["fwd_tiles"] / steps
+    return {"workload": "c5", "ms_per_step": wall_ms, "fwd_ms": f_ms, "fwd_tflops": F / f_ms / 1e9, "fwd_flops": F,
+            "merge_ms": m_ms, "merge_bytes": merge_bytes, "merge_gbps": merge_bytes / m_ms / 1e6,
+            "merge_frac_of_hbm": merge_bytes / m_ms / 1e6 / HBM_PEAK_GBPS,
+            "fwd_plus_merge_tflops": F / wall_ms / 1e9}
+
+
+def cpu_baseline():
+    """The reference's block-loop path restated on the CPU (oracle.block_loop_fwd), timed on
+    config 1 exactly: B=1, S=8192, Nh=8, d=128, fp32, 16x16 causal block grid, forward only."""
+    import torch
+    from oracle import attn_oracle as ao
+    from ultraattn_amd import masks
+    mask = masks.config_causal(16)
+    g = torch.Generator().manual_seed(0)
+    q, k, v = (torch.randn(1, 8192, 8, 128, generator=g, dtype=torch.float32) for _ in range(3))
+    F = fwd_flops(mask, nh=8)
+    times = []
+    while len(times) < 4 or (sum(times) < 12.0 and len(times) < 200):     # 1 warm-up, then >= 3 runs, ~12 s of CPU work
+        t0 = time.perf_counter()
+        ao.block_loop_fwd(q, k, v, mask, BLOCK, SCALE)
+        times.append(time.perf_counter() - t0)
+        if sum(times) > 40:
+            break
+    timed = times[1:] or times
+    best = min(timed)
+    return {"value": F / best / 1e12, "unit": "TFLOP/s", "cores": torch.get_num_threads(), "kind": "port",
+            "sample": "config 1 whole: B=1 S=8192 Nh=8 d=128 fp32 causal 16x16 blocks of 512, forward, "
+                      f"{len(timed)} runs, min {best:.3f} s, median {sorted(timed)[len(timed) // 2]:.3f} s",
+            "affinity_cores": len(os.sched_getaffinity(0)), "flops": F}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=10)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--workload", default="c3", choices=["c2", "c3", "c4", "c5"])
+    ap.add_argument("--no-extra", action="store_true", help="skip the other workloads")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    a = ap.parse_args()
+    if a.gpus != 1:
+        sys.exit("bench.py measures one GPU's share of the path: run it with --gpus 1 "
+                 "(no multi-GPU figure exists for this build)")
+    import torch
+    if not torch.cuda.is_available():
+        sys.exit("bench.py needs an MI355X (no CPU fallback for the kernels)")
+    prop = torch.cuda.get_device_properties(0)
+    clock_ghz = getattr(prop, "clock_rate", 2400000) / 1e6
+    peak = prop.multi_processor_count * FLOP_PER_CLK_PER_CU * clock_ghz / 1e3      # TFLOP/s
+    log(f"device {prop.name}: {prop.multi_processor_count} CUs @ {clock_ghz:.2f} GHz -> bf16 MFMA peak {peak:.1f} TFLOP/s")
+
+    if a.workload == "c5":
+        main_res = run_c5(a.steps, a.warmup)
+    else:
+        main_res = run_attention(a.workload, a.steps, a.warmup, backward=a.workload in ("c3", "c4"))
+    log(json.dumps(main_res))
+    backward = "fwd_bwd_tflops" in main_res
+    if backward:
+        kt = time_bwd_kernels(a.workload, max(3, a.steps // 2))
+        F = main_res["fwd_flops"]
+        # dominant kernel: dK/dV.  Algorithmic flops of that launch: 4 of the backward's 5 GEMMs.
+        roof = {"kernel": "dkdv_kernel", "bound": "mfma", "achieved": 2.0 * F / kt["dkdv"] / 1e9, "peak": peak,
+                "unit": "TFLOP/s", "traffic": None, "kernel_ms": kt["dkdv"]}
+        main_res.update(dkdv_ms=kt["dkdv"], dq_ms=kt["dq"], dkdv_tflops=2.0 * F / kt["dkdv"] / 1e9,
+                        dq_tflops=0.5 * F / kt["dq"] / 1e9)
+        value = main_res["fwd_bwd_tflops"]
+        metric = "effective TFLOP/s on active blocks, forward+backward"
+    else:
+        ms = main_res["fwd_ms"]
+        roof = {"kernel": "fwd_kernel", "bound": "mfma", "achieved": main_res["fwd_tflops"], "peak": peak,
+                "unit": "TFLOP/s", "traffic": None, "kernel_ms": ms}
+        value = main_res.get("fwd_plus_merge_tflops", main_res["fwd_tflops"])
+        metric = "effective TFLOP/s on active blocks, forward"
+    roof["frac"] = roof["achieved"] / roof["peak"]
+
+    extra = {}
+    if not a.no_extra:
+        for w in ("c3", "c4", "c2", "c5"):
+            if w == a.workload:
+                continue
+            torch.cuda.empty_cache()
+            r = run_c5(max(3, a.steps // 2), 2) if w == "c5" else \
+                run_attention(w, max(3, a.steps // 2), 2, backward=w in ("c3", "c4"))
+            for key in ("tilelist_sha256", "fwd_flops"):
+                r.pop(key, None)
+            r["fwd_frac_of_peak"] = r["fwd_tflops"] / peak
+            if "fwd_bwd_tflops" in r:
+                r["fwd_bwd_frac_of_peak"] = r["fwd_bwd_tflops"] / peak
+            extra[w] = r
+            log(json.dumps(r))
+    out = {"metric": metric, "value": value, "unit": "TFLOP/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
+           "ms_per_step": main_res["ms_per_step"], "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+           "dtype": "bf16", "data": "synthetic N(0,1) q/k/v/dO from a seeded device generator, random, no weights",
+           "config": {"workload": {"c2": "causal 32k (config 2), forward", "c3": "strided 128k (config 3), forward+backward",
+                                   "c4": "global+local 128k (config 4), forward+backward",
+                                   "c5": "streaming shard 64k x 512k (config 5), 4 forward kernel tiles + merge"}[a.workload],
+                      "batch": 1, "heads": HEADS, "head_dim": 128, "block": BLOCK, "tile": 128,
+                      "seq_q": int(workload_mask(a.workload).shape[0]) * BLOCK,
+                      "seq_kv": int(workload_mask(a.workload).shape[1]) * BLOCK},
+           "frac_of_bf16_mfma_peak": value / peak, "peak_tflops": peak, "detail": main_res,
+           "fwd_frac_of_peak": main_res["fwd_tflops"] / peak, "roofline": roof, "extra": extra}
+    if not a.no_cpu:
+        out["cpu_baseline"] = cpu_baseline()
+        log(json.dumps(out["cpu_baseline"]))
+    print(json.dumps(out), flush=True)
+
+
+if __name__ == "__main__":
+    main()
