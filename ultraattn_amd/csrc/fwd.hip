@@ -1,8 +1,9 @@
 // Block-sparse flash-attention forward for gfx950 (MI355X).
 //
 // One workgroup (4 wavefronts) per (query tile of 128 rows, head).  It walks the query tile's
-// CSR entries; per entry the 128x128 K and V tiles are staged in LDS.  Each wavefront owns 32
-// query rows and computes the TRANSPOSED products
+// CSR entries; each 128x128 K/V tile is streamed as two 64-key half tiles through two LDS
+// stages (A, B) that are filled by asynchronous global->LDS copies while the other stage is
+// being consumed.  Each wavefront owns 32 query rows and computes the TRANSPOSED products
 //     S^T[key, q] = K Q^T      (A = K fragment from LDS, B = Q fragment held in registers)
 //     O^T[d,  q] += V^T P^T    (A = V^T fragment via transposing LDS reads, B = P^T)
 // with v_mfma_f32_32x32x16_bf16.  In the 32x32 accumulator layout a lane holds ONE query
@@ -23,22 +24,135 @@ struct FwdParams {
   int heads_per_xcd;     // batch*n_heads / 8 when divisible, else 0
 };
 
+constexpr int kHalf = 64;                          // keys per pipeline stage
+constexpr int kHalfBytes = kHalf * kRowBytes;      // 16 KiB
+// P is computed against the row's current reference max without looking at the new scores'
+// max; only when a block's row sum shows that some score exceeded the reference by more than
+// ~2^kRaiseLog2 is the reference raised (and O, l rescaled, P recomputed).  O/l stay exact
+// because numerator and denominator always share the reference.
+constexpr float kRaiseSum = 16777216.f;     // 2^24
+
+struct SoftmaxState {
+  float m_run = -INFINITY;   // reference max of the row (log2 domain, scaled)
+  float m_use = 0.f;         // m_run, or 0 while the row has not seen a visible key
+  float l_run = 0.f;         // this half-wave's partial row sum
+};
+
+// One 64-key half tile for this wave's 32 query rows.  With `mask` (wave-uniform) keys beyond
+// the query's own tile-local index are hidden; `key0` = tile-local index of the half's first key.
+__device__ __forceinline__ void half_tile(const unsigned char* sK, const unsigned char* sV, const bf16x8 (&qf)[8],
+                                          f32x16 (&oacc)[4], SoftmaxState& st, const TrLane& tr, float scale_log2,
+                                          int l32, int hi, int q_local, int key0, bool mask, bool first) {
+  // ---- S^T = K Q^T : 2 blocks of 32 keys x 32 queries ------------------------------------
+  f32x16 s[2];
+#pragma unroll
+  for (int mb = 0; mb < 2; ++mb) {
+    s[mb] = f32x16{0};
+#pragma unroll
+    for (int ks = 0; ks < 8; ++ks) {
+      const bf16x8 a = lds_read_b128(sK, lds_off_k(32 * mb + l32, 2 * ks + hi));
+      s[mb] = mfma32(a, qf[ks], s[mb]);
+    }
+  }
+  // element (mb, i) of this lane: key key0 + 32*mb + 8*(i/4) + 4*hi + i%4, query q_local
+  if (mask) {
+#pragma unroll
+    for (int mb = 0; mb < 2; ++mb)
+#pragma unroll
+      for (int i = 0; i < 16; ++i)
+        if (key0 + 32 * mb + 8 * (i >> 2) + 4 * hi + (i & 3) > q_local) s[mb][i] = -INFINITY;
+  }
+  // ---- online softmax (fp32, log2 domain) ---------------------------------------------------
+  float rs = 0.f;
+  bf16x8 pf[4];
+  bool raise = first;
+  if (!first) {
+#pragma unroll
+    for (int mb = 0; mb < 2; ++mb)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        const float pv = fast_exp2(fmaf(s[mb][i], scale_log2, -st.m_use));
+        rs += pv;
+        pf[mb * 2 + (i >> 3)][i & 7] = (bf16)pv;
+      }
+    raise = __builtin_amdgcn_ballot_w64(!(rs < kRaiseSum)) != 0;       // wave-uniform, rare
+  }
+  if (raise) {
+    float mx = fmaxf(s[0][0], s[1][0]);
+#pragma unroll
+    for (int i = 1; i < 16; ++i) mx = fmaxf(mx, fmaxf(s[0][i], s[1][i]));
+    mx = xhalf_max(mx) * scale_log2;
+    const float m_new = fmaxf(st.m_run, mx);
+    const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
+    const float alpha = (m_new == st.m_run) ? 1.f : fast_exp2(st.m_run - m_use);      // m_run = -inf -> 0
+    st.m_run = m_new;
+    st.m_use = m_use;
+    st.l_run *= alpha;
+#pragma unroll
+    for (int mbd = 0; mbd < 4; ++mbd)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) oacc[mbd][i] *= alpha;
+    rs = 0.f;
+#pragma unroll
+    for (int mb = 0; mb < 2; ++mb)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        const float pv = fast_exp2(fmaf(s[mb][i], scale_log2, -m_use));
+        rs += pv;
+        pf[mb * 2 + (i >> 3)][i & 7] = (bf16)pv;
+      }
+  }
+  st.l_run += rs;
+  // ---- O^T += V^T P^T : 4 blocks of 32 d x 32 queries, 4 steps of 16 keys -------------------
+#pragma unroll
+  for (int kk = 0; kk < 4; ++kk)
+#pragma unroll
+    for (int mbd = 0; mbd < 4; ++mbd) {
+      const bf16x8 a = lds_read_tr_frag<lds_off_v>(sV, tr, 16 * kk, mbd);
+      oacc[mbd] = mfma32(a, pf[kk], oacc[mbd]);
+    }
+}
+
 __global__ __launch_bounds__(256, 2) void fwd_kernel(const FwdParams p) {
-  __shared__ __attribute__((aligned(16))) unsigned char smem[2 * kTileBytes];
-  unsigned char* sK = smem;
-  unsigned char* sV = smem + kTileBytes;
+  // two pipeline stages, distinct arrays so that reads of one stage need not wait for the
+  // copies in flight into the other
+  __shared__ __attribute__((aligned(1024))) unsigned char sKA[kHalfBytes];
+  __shared__ __attribute__((aligned(1024))) unsigned char sVA[kHalfBytes];
+  __shared__ __attribute__((aligned(1024))) unsigned char sKB[kHalfBytes];
+  __shared__ __attribute__((aligned(1024))) unsigned char sVB[kHalfBytes];
 
-  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int l32 = lane & 31, hi = lane >> 5;
-
   int pos, bh;
   map_block(blockIdx.x, p.batch * p.n_heads, p.heads_per_xcd, pos, bh);
   const int qt = p.q_order[pos];
   const int b = bh / p.n_heads, h = bh % p.n_heads;
 
+  const bf16* kbase = p.k + b * p.ks.b + h * p.ks.h;
+  const bf16* vbase = p.v + b * p.vs.b + h * p.vs.h;
+  const int e0 = p.row_ptr[qt], e1 = p.row_ptr[qt + 1];
+  const int k_stride = (int)p.ks.s, v_stride = (int)p.vs.s;
+  int koff[4], voff[4];
+  dma_voffsets<lds_off_k, 4>(koff, k_stride, wave, lane);
+  dma_voffsets<lds_off_v, 4>(voff, v_stride, wave, lane);
+  const int k_half = kHalf * k_stride * 2, v_half = kHalf * v_stride * 2;                 // bytes
+  const uint32_t k_extent = (uint32_t)((kTile - 1) * k_stride + kHeadDim) * 2;            // bytes of one tile
+  const uint32_t v_extent = (uint32_t)((kTile - 1) * v_stride + kHeadDim) * 2;
+  auto k_rsrc = [&](int kt) { return make_rsrc(kbase + (int64_t)kt * kTile * k_stride, k_extent); };
+  auto v_rsrc = [&](int kt) { return make_rsrc(vbase + (int64_t)kt * kTile * v_stride, v_extent); };
+
+  // first half tile of the first entry goes in flight before anything else
+  int kt = e0 < e1 ? min(max(p.col_idx[e0], 0), p.n_ktiles - 1) : 0;
+  if (e0 < e1) {
+    dma_half_tile_buf<4>(sKA, k_rsrc(kt), koff, 0, wave);
+    dma_half_tile_buf<4>(sVA, v_rsrc(kt), voff, 0, wave);
+  }
+
   // Q fragment (B operand of S^T): lane holds query row 32*wave + lane%32,
   // d = 16*ks + 8*(lane/32) .. +7 for ks = 0..7.
-  const int qrow = qt * kTile + wave * 32 + l32;
+  const int q_local = wave * 32 + l32;
+  const int qrow = qt * kTile + q_local;
   const bf16* qp = p.q + b * p.qs.b + (int64_t)qrow * p.qs.s + h * p.qs.h + hi * 8;
   bf16x8 qf[8];
 #pragma unroll
@@ -47,87 +161,34 @@ __global__ __launch_bounds__(256, 2) void fwd_kernel(const FwdParams p) {
   f32x16 oacc[4];
 #pragma unroll
   for (int i = 0; i < 4; ++i) oacc[i] = f32x16{0};
-  float m_run = -INFINITY;   // running row max, log2 domain (already scaled)
-  float l_run = 0.f;         // this half-wave's partial row sum
-
-  const bf16* kbase = p.k + b * p.ks.b + h * p.ks.h;
-  const bf16* vbase = p.v + b * p.vs.b + h * p.vs.h;
-  const int e0 = p.row_ptr[qt], e1 = p.row_ptr[qt + 1];
-
+  SoftmaxState st;
   const TrLane tr(lane);
 
   for (int e = e0; e < e1; ++e) {
-    const int kt = p.col_idx[e];
     const int causal = p.flag[e];
-    if ((unsigned)kt >= (unsigned)p.n_ktiles) continue;   // uniform: never index outside K/V
+    const int kt_next = e + 1 < e1 ? min(max(p.col_idx[e + 1], 0), p.n_ktiles - 1) : kt;
+    // stage A (keys 0..63 of this tile) has landed; everyone is done with stage B
+    wait_vmem_all();
     __syncthreads();
-    stage_tile<lds_off_k>(sK, kbase + (int64_t)kt * kTile * p.ks.s, p.ks.s, tid);
-    stage_tile<lds_off_v>(sV, vbase + (int64_t)kt * kTile * p.vs.s, p.vs.s, tid);
+    dma_half_tile_buf<4>(sKB, k_rsrc(kt), koff, k_half, wave);
+    dma_half_tile_buf<4>(sVB, v_rsrc(kt), voff, v_half, wave);
+    // causal tile: queries 64..127 (waves 2, 3) see all of keys 0..63
+    half_tile(sKA, sVA, qf, oacc, st, tr, p.scale_log2, l32, hi, q_local, 0, causal && wave < 2, e == e0);
+    // stage B has landed; everyone is done with stage A
+    wait_vmem_all();
     __syncthreads();
-
-    // ---- S^T = K Q^T : 4 blocks of 32 keys x 32 queries --------------------------------
-    f32x16 s[4];
-#pragma unroll
-    for (int mb = 0; mb < 4; ++mb) {
-      s[mb] = f32x16{0};
-#pragma unroll
-      for (int ks = 0; ks < 8; ++ks) {
-        bf16x8 a = lds_read_b128(sK, lds_off_k(32 * mb + l32, 2 * ks + hi));
-        s[mb] = mfma32(a, qf[ks], s[mb]);
-      }
+    if (e + 1 < e1) {
+      dma_half_tile_buf<4>(sKA, k_rsrc(kt_next), koff, 0, wave);
+      dma_half_tile_buf<4>(sVA, v_rsrc(kt_next), voff, 0, wave);
     }
-    // element (mb, i) of this lane: key 32*mb + 8*(i/4) + 4*hi + i%4, query 32*wave + l32
-    if (causal) {
-      const int ql = wave * 32 + l32;
-#pragma unroll
-      for (int mb = 0; mb < 4; ++mb)
-#pragma unroll
-        for (int i = 0; i < 16; ++i) {
-          const int key = 32 * mb + 8 * (i >> 2) + 4 * hi + (i & 3);
-          if (key > ql) s[mb][i] = -INFINITY;
-        }
-    }
-    // ---- online softmax (fp32, log2 domain) ---------------------------------------------
-    float mx = -INFINITY;
-#pragma unroll
-    for (int mb = 0; mb < 4; ++mb)
-#pragma unroll
-      for (int i = 0; i < 16; ++i) mx = fmaxf(mx, s[mb][i]);
-    mx = xhalf_max(mx) * p.scale_log2;
-    const float m_new = fmaxf(m_run, mx);
-    const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
-    const float alpha = fast_exp2(m_run - m_use);
-    m_run = m_new;
-    float rs = 0.f;
-    bf16x8 pf[8];
-#pragma unroll
-    for (int mb = 0; mb < 4; ++mb) {
-#pragma unroll
-      for (int i = 0; i < 16; ++i) {
-        const float pv = fast_exp2(fmaf(s[mb][i], p.scale_log2, -m_use));
-        rs += pv;
-        pf[mb * 2 + (i >> 3)][i & 7] = (bf16)pv;
-      }
-    }
-    l_run = l_run * alpha + rs;
-#pragma unroll
-    for (int mbd = 0; mbd < 4; ++mbd)
-#pragma unroll
-      for (int i = 0; i < 16; ++i) oacc[mbd][i] *= alpha;
-
-    // ---- O^T += V^T P^T : 4 blocks of 32 d x 32 queries, 8 steps of 16 keys ----------------
-#pragma unroll
-    for (int kk = 0; kk < 8; ++kk) {
-#pragma unroll
-      for (int mbd = 0; mbd < 4; ++mbd) {
-        const bf16x8 a = lds_read_tr_frag<lds_off_v>(sV, tr, 16 * kk, mbd);
-        oacc[mbd] = mfma32(a, pf[kk], oacc[mbd]);
-      }
-    }
+    // causal tile: queries 0..63 (waves 0, 1) see none of keys 64..127
+    if (!causal || wave >= 2)
+      half_tile(sKB, sVB, qf, oacc, st, tr, p.scale_log2, l32, hi, q_local, kHalf, causal, false);
+    kt = kt_next;
   }
 
   // ---- epilogue: normalise, write O (bf16) and LSE (natural log) -------------------------
-  const float l_tot = xhalf_sum(l_run);
+  const float l_tot = xhalf_sum(st.l_run);
   const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
   bf16* op = p.o + b * p.os.b + (int64_t)qrow * p.os.s + h * p.os.h;
 #pragma unroll
@@ -140,7 +201,7 @@ __global__ __launch_bounds__(256, 2) void fwd_kernel(const FwdParams p) {
       *reinterpret_cast<bf16x4*>(op + 32 * mbd + 8 * g + 4 * hi) = w;
     }
   if (hi == 0) {
-    const float lse = l_tot > 0.f ? (m_run + __builtin_amdgcn_logf(l_tot)) * kLn2 : -INFINITY;
+    const float lse = l_tot > 0.f ? (st.m_run + __builtin_amdgcn_logf(l_tot)) * kLn2 : -INFINITY;
     p.lse[((int64_t)b * p.n_heads + h) * ((int64_t)p.n_qtiles * kTile) + qrow] = lse;
   }
 }
@@ -162,6 +223,7 @@ extern "C" int ua_bsa_fwd(const void* q, const void* k, const void* v, void* o, 
   if (!aligned16(q) || !aligned16(k) || !aligned16(v) || !aligned16(o)) return UA_ERR_ALIGN;
   if (!strides_ok(q_strides) || !strides_ok(k_strides) || !strides_ok(v_strides) || !strides_ok(o_strides))
     return UA_ERR_ALIGN;
+  if (k_strides[1] > (INT32_MAX >> 9) || v_strides[1] > (INT32_MAX >> 9)) return UA_ERR_SHAPE;
   if (int rc = check_device()) return rc;
   FwdParams p;
   p.q = (const bf16*)q; p.k = (const bf16*)k; p.v = (const bf16*)v; p.o = (bf16*)o; p.lse = lse;

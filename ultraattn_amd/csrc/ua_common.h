@@ -100,6 +100,61 @@ __device__ __forceinline__ bf16x8 lds_read_tr_frag(const unsigned char* smem, co
   return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
 }
 
+// Asynchronous global -> LDS copy of 16 bytes per lane (global_load_lds_dwordx4): the wave's 64
+// lanes fill 1 KiB starting at the wave-uniform LDS address `lds_dst`, lane l at +16*l, each
+// from its own global address.  Completion is tracked by vmcnt.
+__device__ __forceinline__ void dma16(const bf16* gsrc, unsigned char* lds_dst) {
+  __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)gsrc,
+                                   (__attribute__((address_space(3))) void*)lds_dst, 16, 0, 0);
+}
+__device__ __forceinline__ void wait_vmem_all() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
+
+// Per-thread source offsets (in elements) for staging a [64][128] bf16 half tile (16 KiB) with
+// NW waves: each thread issues 16/NW DMA instructions; instruction i of wave w fills LDS rows
+// 4*(NW*i + w) .. +3; lane l lands in that group's row l/16, physical 16-byte slot l%16, so
+// it must fetch the logical chunk that the XOR layout `OFF` maps to that slot.
+template <int (*OFF)(int, int), int NW>
+__device__ __forceinline__ void dma_offsets(int (&off)[16 / NW], int64_t row_stride, int wave, int lane) {
+#pragma unroll
+  for (int i = 0; i < 16 / NW; ++i) {
+    const int r = 4 * (NW * i + wave) + (lane >> 4);
+    const int phys = lane & 15;
+    const int c = ((OFF(r, 0) - r * kRowBytes) >> 4) ^ phys;
+    off[i] = (int)(r * row_stride) + c * 8;
+  }
+}
+template <int NW>
+__device__ __forceinline__ void dma_half_tile(unsigned char* lds, const bf16* g, const int (&off)[16 / NW], int wave) {
+#pragma unroll
+  for (int i = 0; i < 16 / NW; ++i) dma16(g + off[i], lds + (NW * i + wave) * 1024);
+}
+
+// Buffer-addressed variant (buffer_load_dwordx4 ... lds): the source address is
+// descriptor base + per-lane byte offset `voff` + wave-uniform byte offset `soff`, so a tile's
+// address arithmetic stays on the scalar unit; reads beyond the descriptor's extent return 0.
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* base, uint32_t bytes) {
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, bytes, 0x00020000);
+}
+__device__ __forceinline__ void dma16_buf(__amdgpu_buffer_rsrc_t r, unsigned char* lds_dst, int voff, int soff) {
+  __builtin_amdgcn_raw_ptr_buffer_load_lds(r, (__attribute__((address_space(3))) void*)lds_dst, 16, voff, soff, 0, 0);
+}
+// Per-thread byte offsets for staging a [64][128] bf16 half tile with NW waves (see dma_offsets).
+template <int (*OFF)(int, int), int NW>
+__device__ __forceinline__ void dma_voffsets(int (&off)[16 / NW], int row_stride, int wave, int lane) {
+#pragma unroll
+  for (int i = 0; i < 16 / NW; ++i) {
+    const int r = 4 * (NW * i + wave) + (lane >> 4);
+    const int c = ((OFF(r, 0) - r * kRowBytes) >> 4) ^ (lane & 15);
+    off[i] = (r * row_stride + c * 8) * 2;
+  }
+}
+template <int NW>
+__device__ __forceinline__ void dma_half_tile_buf(unsigned char* lds, __amdgpu_buffer_rsrc_t r, const int (&voff)[16 / NW],
+                                                  int soff, int wave) {
+#pragma unroll
+  for (int i = 0; i < 16 / NW; ++i) dma16_buf(r, lds + (NW * i + wave) * 1024, voff[i], soff);
+}
+
 // blockIdx -> (position in the launch order, batch*head).  Consecutive workgroups go to
 // consecutive XCDs; each XCD gets its own heads so that tiles which share operands meet in
 // one L2.  heads_per_xcd = batch*n_heads/8 when divisible, else 0 (plain mapping).
