@@ -19,7 +19,8 @@
  *    the transposed CSC over key tiles.  flag 0 = full tile, 1 = causal tile (key j visible to
  *    query i iff j <= i on tile-local indices; such tiles sit on the mask's diagonal,
  *    orchestrated_attn/orchestrated_attn_impl.py:91).  `*_order` is a permutation of the tile
- *    rows (columns) giving the launch order, longest first.
+ *    rows (columns) giving the launch order: rows much longer than average first, the rest in
+ *    lexicographic order of their index lists so that rows sharing K/V tiles run together.
  *  - Every function returns 0 (UA_OK) or a negative UA_ERR_* code; ua_strerror() names it.
  *    No exceptions cross this boundary and nothing aborts.
  *  - Functions hold no mutable global state and may be called from several host threads on
@@ -60,7 +61,7 @@ const char *ua_strerror(int rc);
  * ua_tilelist_build fills caller-allocated HOST arrays:
  *   row_ptr[n_qtiles+1], col_idx[nnz], flag[nnz]      CSR over query tiles
  *   col_ptr[n_ktiles+1], row_idx[nnz], cflag[nnz]     CSC over key tiles
- *   q_order[n_qtiles], k_order[n_ktiles]              longest-first stable orders           */
+ *   q_order[n_qtiles], k_order[n_ktiles]              launch orders                         */
 int ua_tilelist_size(const uint8_t *block_mask, int n_qblocks, int n_kblocks, int rate,
                      int64_t *n_qtiles, int64_t *n_ktiles, int64_t *nnz);
 int ua_tilelist_build(const uint8_t *block_mask, int n_qblocks, int n_kblocks, int rate,

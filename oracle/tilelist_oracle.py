@@ -124,12 +124,28 @@ def build_tile_list(block_table: np.ndarray, rate: int) -> Dict[str, np.ndarray]
     for _, l, _ in by_col:
         col_ptr[l + 1] += 1
     col_ptr = np.cumsum(col_ptr, dtype=np.int64).astype(np.int32)
-    qlen = np.diff(row_ptr)
-    klen = np.diff(col_ptr)
-    q_order = np.array(sorted(range(nqt), key=lambda i: (-int(qlen[i]), i)), dtype=np.int32).reshape(-1)
-    k_order = np.array(sorted(range(nkt), key=lambda i: (-int(klen[i]), i)), dtype=np.int32).reshape(-1)
+    q_order = launch_order(row_ptr, col_idx)
+    k_order = launch_order(col_ptr, row_idx)
     return dict(row_ptr=row_ptr, col_idx=col_idx, flag=flag, col_ptr=col_ptr, row_idx=row_idx,
                 cflag=cflag, q_order=q_order, k_order=k_order, n_qtiles=nqt, n_ktiles=nkt)
+
+
+def launch_order(ptr: np.ndarray, idx: np.ndarray) -> np.ndarray:
+    """Launch order of the rows of a CSR (or columns of a CSC).  Rows much longer than average
+    (length * n_rows > 2 * nnz) come first, longest first, so that they cannot end up as the
+    tail of the launch; all other rows follow in lexicographic order of their index lists
+    (a list that is a prefix of another sorts after it), which puts rows that walk the same
+    K/V tiles next to each other.  Ties by row number."""
+    n = len(ptr) - 1
+    nnz = int(ptr[-1])
+    inf = 1 << 40
+
+    def key(i):
+        lst = tuple(int(x) for x in idx[ptr[i]:ptr[i + 1]])
+        if len(lst) * n > 2 * nnz:
+            return (0, (-len(lst),), i)
+        return (1, lst + (inf,), i)
+    return np.array(sorted(range(n), key=key), dtype=np.int32).reshape(-1)
 
 
 def tiles_to_element_mask(tl: Dict[str, np.ndarray], tile: int) -> np.ndarray:

@@ -52,10 +52,30 @@ def test_full_size_digests(golden_dir, lib):
         pairs = sorted((int(c), r) for r in range(tl.n_qtiles) for c in tl.col_idx[tl.row_ptr[r]:tl.row_ptr[r + 1]])
         csc = [(c, int(r)) for c in range(tl.n_ktiles) for r in tl.row_idx[tl.col_ptr[c]:tl.col_ptr[c + 1]]]
         assert pairs == csc
-        # orders are permutations sorted by length, longest first, ties by index
-        ql = np.diff(tl.row_ptr)
+        # launch orders are permutations; rows much longer than average lead, longest first
         assert sorted(tl.q_order.tolist()) == list(range(tl.n_qtiles))
-        assert all((ql[a], -a) >= (ql[b], -b) for a, b in zip(tl.q_order[:-1], tl.q_order[1:]))
+        assert sorted(tl.k_order.tolist()) == list(range(tl.n_ktiles))
+        ql = np.diff(tl.row_ptr)
+        n_long = int((ql * tl.n_qtiles > 2 * tl.nnz).sum())
+        head = tl.q_order[:n_long]
+        assert all(ql[r] * tl.n_qtiles > 2 * tl.nnz for r in head)
+        assert all(ql[a] >= ql[b] for a, b in zip(head[:-1], head[1:]))
+
+
+def test_launch_order_groups_rows_with_common_tiles(lib):
+    """Independent statement of the order: plain Python sort of the padded index lists."""
+    m = masks.config_strided(32)
+    tl = build_tile_list(m, block=256)
+    lists = [tuple(tl.col_idx[tl.row_ptr[r]:tl.row_ptr[r + 1]]) for r in range(tl.n_qtiles)]
+    assert not any(len(l) * tl.n_qtiles > 2 * tl.nnz for l in lists)
+    want = sorted(range(tl.n_qtiles), key=lambda r: (lists[r] + (10 ** 9,), r))
+    assert tl.q_order.tolist() == want
+    # the two query tiles of one strided block sit next to each other
+    pos = {r: i for i, r in enumerate(tl.q_order.tolist())}
+    assert all(abs(pos[2 * b] - pos[2 * b + 1]) == 1 for b in range(32))
+    # global rows of the global+local mask are the long ones and come first
+    tg = build_tile_list(masks.config_global_local(64, 2, 4), block=128)
+    assert sorted(tg.q_order[:2].tolist()) == [0, 1]
 
 
 def test_causal_flag_and_offset(lib):

@@ -44,18 +44,107 @@ __device__ __forceinline__ void store_acc_t(bf16* row_ptr, const f32x16 (&acc)[4
     }
 }
 
-__global__ __launch_bounds__(256, 1) void dkdv_kernel(const BwdParams p) {
-  __shared__ __attribute__((aligned(16))) unsigned char smem[2 * kTileBytes + 2 * kTile * 4];
-  unsigned char* sQ = smem;
-  unsigned char* sdO = smem + kTileBytes;
-  float* sLse = reinterpret_cast<float*>(smem + 2 * kTileBytes);
-  float* sDelta = sLse + kTile;
+constexpr int kHalf = 64;
+constexpr int kHalfBytes = kHalf * kRowBytes;      // 16 KiB
 
-  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+// Stage one full [128][128] bf16 tile (two half tiles) with asynchronous copies, 256 threads.
+__device__ __forceinline__ void dma_tile_buf(unsigned char* lds, __amdgpu_buffer_rsrc_t r, const int (&voff)[4],
+                                             int half_bytes, int wave) {
+  dma_half_tile_buf<4>(lds, r, voff, 0, wave);
+  dma_half_tile_buf<4>(lds + kHalfBytes, r, voff, half_bytes, wave);
+}
+
+// Per-lane LDS byte offsets into a tile held in the universal layout, for the first 32-row
+// block; later blocks add 32*kRowBytes per block (the XOR term repeats every 16 rows).
+struct LaneOffsU {
+  int nat[8];      // 128-bit row-fragment reads: row lane%32, chunk 2*ks + lane/32
+  int tr[4][2];    // transposing reads for d-block mbd: rows row_in (+8)
+  __device__ __forceinline__ LaneOffsU(int l32, int hi, const TrLane& t) {
+#pragma unroll
+    for (int ks = 0; ks < 8; ++ks) nat[ks] = lds_off_u(l32, 2 * ks + hi);
+#pragma unroll
+    for (int mbd = 0; mbd < 4; ++mbd) {
+      tr[mbd][0] = lds_off_u(t.row_in, 4 * mbd + t.chunk_in) + t.sub;
+      tr[mbd][1] = lds_off_u(t.row_in + 8, 4 * mbd + t.chunk_in) + t.sub;
+    }
+  }
+};
+__device__ __forceinline__ bf16x8 read_tr_pair(const unsigned char* smem, int off_lo, int off_hi) {
+  const bf16x4 a = lds_read_tr16_b64(smem, off_lo);
+  const bf16x4 b = lds_read_tr16_b64(smem, off_hi);
+  return __builtin_shufflevector(a, b, 0, 1, 2, 3, 4, 5, 6, 7);
+}
+
+// dK/dV: per query tile of the column, for each block of 32 query rows.
+__device__ __forceinline__ void dkdv_tile(const unsigned char* sQ, const unsigned char* sdO, const float* sLse,
+                                          const float* sDelta, const bf16x8 (&kf)[8], const bf16x8 (&vf)[8],
+                                          f32x16 (&dk)[4], f32x16 (&dv)[4], const LaneOffsU& lo, float scale_log2,
+                                          int hi, int key_l, bool causal) {
+#pragma unroll 1
+  for (int nb = 0; nb < 4; ++nb) {     // 32 query rows at a time
+    // this block's per-lane offsets: 16 adds; everything else is an immediate offset
+    const int blk = nb * 32 * kRowBytes;
+    int nat[8], trb[4][2];
+#pragma unroll
+    for (int ks = 0; ks < 8; ++ks) nat[ks] = lo.nat[ks] + blk;
+#pragma unroll
+    for (int mbd = 0; mbd < 4; ++mbd) { trb[mbd][0] = lo.tr[mbd][0] + blk; trb[mbd][1] = lo.tr[mbd][1] + blk; }
+    f32x16 s = f32x16{0}, dp = f32x16{0};
+#pragma unroll
+    for (int ks = 0; ks < 8; ++ks) {
+      const bf16x8 aq = lds_read_b128(sQ, nat[ks]);
+      s = mfma32(aq, kf[ks], s);
+      const bf16x8 ad = lds_read_b128(sdO, nat[ks]);
+      dp = mfma32(ad, vf[ks], dp);
+    }
+    // element i: query row 32*nb + 8*(i/4) + 4*hi + i%4, key column key_l
+    if (causal) {
+#pragma unroll
+      for (int i = 0; i < 16; ++i)
+        if (key_l > 32 * nb + 8 * (i >> 2) + 4 * hi + (i & 3)) s[i] = -INFINITY;
+    }
+    bf16x8 pb[2], dsb[2];
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+      const int q0 = 32 * nb + 8 * g + 4 * hi;
+      const f32x4 l4 = *reinterpret_cast<const f32x4*>(sLse + q0);
+      const f32x4 d4 = *reinterpret_cast<const f32x4*>(sDelta + q0);
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int i = 4 * g + j;
+        const float pv = fast_exp2(fmaf(s[i], scale_log2, -l4[j]));
+        const float dsv = pv * (dp[i] - d4[j]);
+        pb[i >> 3][i & 7] = (bf16)pv;
+        dsb[i >> 3][i & 7] = (bf16)dsv;
+      }
+    }
+#pragma unroll
+    for (int t = 0; t < 2; ++t)
+#pragma unroll
+      for (int mbd = 0; mbd < 4; ++mbd) {
+        const bf16x8 a_do = read_tr_pair(sdO + 16 * t * kRowBytes, trb[mbd][0], trb[mbd][1]);
+        dv[mbd] = mfma32(a_do, pb[t], dv[mbd]);
+        const bf16x8 a_q = read_tr_pair(sQ + 16 * t * kRowBytes, trb[mbd][0], trb[mbd][1]);
+        dk[mbd] = mfma32(a_q, dsb[t], dk[mbd]);
+      }
+  }
+}
+
+__global__ __launch_bounds__(256, 1) void dkdv_kernel(const BwdParams p) {
+  // two stages (Q tile, dO tile, the rows' lse and delta), distinct arrays per stage
+  __shared__ __attribute__((aligned(1024))) unsigned char sQ0[kTileBytes];
+  __shared__ __attribute__((aligned(1024))) unsigned char sdO0[kTileBytes];
+  __shared__ __attribute__((aligned(1024))) unsigned char sQ1[kTileBytes];
+  __shared__ __attribute__((aligned(1024))) unsigned char sdO1[kTileBytes];
+  __shared__ __attribute__((aligned(16))) float sStat0[2 * kTile];
+  __shared__ __attribute__((aligned(16))) float sStat1[2 * kTile];
+
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int l32 = lane & 31, hi = lane >> 5;
   int pos, bh;
   map_block(blockIdx.x, p.batch * p.n_heads, p.heads_per_xcd, pos, bh);
-  const int kt = p.order[pos];
+  const int kt = sload(p.order, pos);
   const int b = bh / p.n_heads, h = bh % p.n_heads;
   const int64_t seq_q = (int64_t)p.n_qtiles * kTile;
 
@@ -78,80 +167,136 @@ __global__ __launch_bounds__(256, 1) void dkdv_kernel(const BwdParams p) {
   const float* lse_row = p.lse + ((int64_t)b * p.n_heads + h) * seq_q;
   const float* delta_row = p.delta + ((int64_t)b * p.n_heads + h) * seq_q;
   const TrLane tr(lane);
+  const LaneOffsU lo(l32, hi, tr);
   const int key_l = wave * 32 + l32;
 
-  const int e0 = p.ptr[kt], e1 = p.ptr[kt + 1];
-  for (int e = e0; e < e1; ++e) {
-    const int qt = p.idx[e];
-    const int causal = p.flag[e];
-    if ((unsigned)qt >= (unsigned)p.n_qtiles) continue;
-    __syncthreads();
-    stage_tile<lds_off_u>(sQ, qbase + (int64_t)qt * kTile * p.qs.s, p.qs.s, tid);
-    stage_tile<lds_off_u>(sdO, dobase + (int64_t)qt * kTile * p.ds.s, p.ds.s, tid);
-    if (tid < kTile) {
-      const float l = lse_row[qt * kTile + tid];
-      sLse[tid] = (l == -INFINITY) ? INFINITY : l * kLog2e;   // rows without keys give P = 0
-    } else {
-      sDelta[tid - kTile] = delta_row[qt * kTile + tid - kTile];
-    }
-    __syncthreads();
+  const int q_stride = (int)p.qs.s, do_stride = (int)p.ds.s;
+  int qoff[4], dooff[4];
+  dma_voffsets<lds_off_u, 4>(qoff, q_stride, wave, lane);
+  dma_voffsets<lds_off_u, 4>(dooff, do_stride, wave, lane);
+  const int q_half = kHalf * q_stride * 2, do_half = kHalf * do_stride * 2;
+  const uint32_t q_extent = (uint32_t)((kTile - 1) * q_stride + kHeadDim) * 2;
+  const uint32_t do_extent = (uint32_t)((kTile - 1) * do_stride + kHeadDim) * 2;
+  auto qtile = [&](int e) { return min(max(sload(p.idx, e), 0), p.n_qtiles - 1); };
+  // rows' statistics: threads 0..127 carry lse (pre-multiplied by log2 e; -inf -> +inf so that
+  // rows without keys give P = 0), threads 128..255 carry delta
+  auto load_stat = [&](int qt) {
+    const float x = tid < kTile ? lse_row[qt * kTile + tid] : delta_row[qt * kTile + tid - kTile];
+    return tid < kTile ? (x == -INFINITY ? INFINITY : x * kLog2e) : x;
+  };
+  auto stage = [&](int qt, unsigned char* sQ, unsigned char* sdO) {
+    dma_tile_buf(sQ, make_rsrc(qbase + (int64_t)qt * kTile * q_stride, q_extent), qoff, q_half, wave);
+    dma_tile_buf(sdO, make_rsrc(dobase + (int64_t)qt * kTile * do_stride, do_extent), dooff, do_half, wave);
+  };
 
-#pragma unroll 1
-    for (int nb = 0; nb < 4; ++nb) {     // 32 query rows at a time
-      f32x16 s = f32x16{0}, dp = f32x16{0};
-#pragma unroll
-      for (int ks = 0; ks < 8; ++ks) {
-        const bf16x8 aq = lds_read_b128(sQ, lds_off_u(32 * nb + l32, 2 * ks + hi));
-        s = mfma32(aq, kf[ks], s);
-        const bf16x8 ad = lds_read_b128(sdO, lds_off_u(32 * nb + l32, 2 * ks + hi));
-        dp = mfma32(ad, vf[ks], dp);
-      }
-      // element i: query row 32*nb + 8*(i/4) + 4*hi + i%4, key column key_l
-      bf16x8 pb[2], dsb[2];
-#pragma unroll
-      for (int g = 0; g < 4; ++g) {
-        const int q0 = 32 * nb + 8 * g + 4 * hi;
-        const f32x4 l4 = *reinterpret_cast<const f32x4*>(sLse + q0);
-        const f32x4 d4 = *reinterpret_cast<const f32x4*>(sDelta + q0);
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-          const int i = 4 * g + j;
-          float pv = fast_exp2(fmaf(s[i], p.scale_log2, -l4[j]));
-          if (causal && key_l > q0 + j) pv = 0.f;
-          const float dsv = pv * (dp[i] - d4[j]);
-          pb[i >> 3][i & 7] = (bf16)pv;
-          dsb[i >> 3][i & 7] = (bf16)dsv;
-        }
-      }
-#pragma unroll
-      for (int t = 0; t < 2; ++t)
-#pragma unroll
-        for (int mbd = 0; mbd < 4; ++mbd) {
-          const bf16x8 a_do = lds_read_tr_frag<lds_off_u>(sdO, tr, 32 * nb + 16 * t, mbd);
-          dv[mbd] = mfma32(a_do, pb[t], dv[mbd]);
-          const bf16x8 a_q = lds_read_tr_frag<lds_off_u>(sQ, tr, 32 * nb + 16 * t, mbd);
-          dk[mbd] = mfma32(a_q, dsb[t], dk[mbd]);
-        }
+  const int e0 = sload(p.ptr, kt), e1 = sload(p.ptr, kt + 1);
+  if (e0 < e1) {
+    const int qt = qtile(e0);
+    sStat0[tid] = load_stat(qt);
+    stage(qt, sQ0, sdO0);
+  }
+  // entries are taken two at a time: even ones through stage 0, odd ones through stage 1
+  for (int e = e0; e < e1; e += 2) {
+    const bool has1 = e + 1 < e1, has2 = e + 2 < e1;
+    float stat = 0.f;
+    wait_vmem_all();
+    __syncthreads();                       // stage 0 landed; everyone is done with stage 1
+    if (has1) {
+      const int qt = qtile(e + 1);
+      stat = load_stat(qt);
+      stage(qt, sQ1, sdO1);
     }
+    dkdv_tile(sQ0, sdO0, sStat0, sStat0 + kTile, kf, vf, dk, dv, lo, p.scale_log2, hi, key_l, sload(p.flag, e) != 0);
+    if (!has1) break;
+    sStat1[tid] = stat;
+    wait_vmem_all();
+    __syncthreads();                       // stage 1 landed; everyone is done with stage 0
+    if (has2) {
+      const int qt = qtile(e + 2);
+      stat = load_stat(qt);
+      stage(qt, sQ0, sdO0);
+    }
+    dkdv_tile(sQ1, sdO1, sStat1, sStat1 + kTile, kf, vf, dk, dv, lo, p.scale_log2, hi, key_l, sload(p.flag, e + 1) != 0);
+    if (has2) sStat0[tid] = stat;
   }
   store_acc_t(p.out0 + b * p.o0s.b + (int64_t)krow * p.o0s.s + h * p.o0s.h, dk, p.scale, hi);
   store_acc_t(p.out1 + b * p.o1s.b + (int64_t)krow * p.o1s.s + h * p.o1s.h, dv, 1.f, hi);
 }
 
-__global__ __launch_bounds__(256, 2) void dq_kernel(const BwdParams p) {
-  __shared__ __attribute__((aligned(16))) unsigned char smem[2 * kTileBytes];
-  unsigned char* sK = smem;
-  unsigned char* sV = smem + kTileBytes;
+// dQ: one 64-key half tile for this wave's 32 query rows.
+__device__ __forceinline__ void dq_half_tile(const unsigned char* sK, const unsigned char* sV, const bf16x8 (&qf)[8],
+                                             const bf16x8 (&dof)[8], f32x16 (&dq)[4], const TrLane& tr,
+                                             float scale_log2, float lse2, float delta, int l32, int hi, int q_l,
+                                             int key0, bool mask) {
+#pragma unroll
+  for (int mb = 0; mb < 2; ++mb) {     // 32 keys at a time
+    f32x16 s = f32x16{0}, dp = f32x16{0};
+#pragma unroll
+    for (int ks = 0; ks < 8; ++ks) {
+      const bf16x8 ak = lds_read_b128(sK, lds_off_u(32 * mb + l32, 2 * ks + hi));
+      s = mfma32(ak, qf[ks], s);
+      const bf16x8 av = lds_read_b128(sV, lds_off_k(32 * mb + l32, 2 * ks + hi));
+      dp = mfma32(av, dof[ks], dp);
+    }
+    // element i: key key0 + 32*mb + 8*(i/4) + 4*hi + i%4, query column q_l
+    if (mask) {
+#pragma unroll
+      for (int i = 0; i < 16; ++i)
+        if (key0 + 32 * mb + 8 * (i >> 2) + 4 * hi + (i & 3) > q_l) s[i] = -INFINITY;
+    }
+    bf16x8 dsb[2];
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      const float pv = fast_exp2(fmaf(s[i], scale_log2, -lse2));
+      dsb[i >> 3][i & 7] = (bf16)(pv * (dp[i] - delta));
+    }
+#pragma unroll
+    for (int t = 0; t < 2; ++t)
+#pragma unroll
+      for (int mbd = 0; mbd < 4; ++mbd) {
+        const bf16x8 a_k = lds_read_tr_frag<lds_off_u>(sK, tr, 32 * mb + 16 * t, mbd);
+        dq[mbd] = mfma32(a_k, dsb[t], dq[mbd]);
+      }
+  }
+}
 
-  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+__global__ __launch_bounds__(256, 2) void dq_kernel(const BwdParams p) {
+  __shared__ __attribute__((aligned(1024))) unsigned char sKA[kHalfBytes];
+  __shared__ __attribute__((aligned(1024))) unsigned char sVA[kHalfBytes];
+  __shared__ __attribute__((aligned(1024))) unsigned char sKB[kHalfBytes];
+  __shared__ __attribute__((aligned(1024))) unsigned char sVB[kHalfBytes];
+
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int l32 = lane & 31, hi = lane >> 5;
   int pos, bh;
   map_block(blockIdx.x, p.batch * p.n_heads, p.heads_per_xcd, pos, bh);
-  const int qt = p.order[pos];
+  const int qt = sload(p.order, pos);
   const int b = bh / p.n_heads, h = bh % p.n_heads;
   const int64_t seq_q = (int64_t)p.n_qtiles * kTile;
 
-  const int qrow = qt * kTile + wave * 32 + l32;
+  const bf16* kbase = p.k + b * p.ks.b + h * p.ks.h;
+  const bf16* vbase = p.v + b * p.vs.b + h * p.vs.h;
+  const int k_stride = (int)p.ks.s, v_stride = (int)p.vs.s;
+  int koff[4], voff[4];
+  dma_voffsets<lds_off_u, 4>(koff, k_stride, wave, lane);
+  dma_voffsets<lds_off_k, 4>(voff, v_stride, wave, lane);
+  const int k_half = kHalf * k_stride * 2, v_half = kHalf * v_stride * 2;
+  const uint32_t k_extent = (uint32_t)((kTile - 1) * k_stride + kHeadDim) * 2;
+  const uint32_t v_extent = (uint32_t)((kTile - 1) * v_stride + kHeadDim) * 2;
+  auto k_rsrc = [&](int kt) { return make_rsrc(kbase + (int64_t)kt * kTile * k_stride, k_extent); };
+  auto v_rsrc = [&](int kt) { return make_rsrc(vbase + (int64_t)kt * kTile * v_stride, v_extent); };
+  auto ktile = [&](int e) { return min(max(sload(p.idx, e), 0), p.n_ktiles - 1); };
+
+  const int e0 = sload(p.ptr, qt), e1 = sload(p.ptr, qt + 1);
+  int kt = e0 < e1 ? ktile(e0) : 0;
+  if (e0 < e1) {
+    dma_half_tile_buf<4>(sKA, k_rsrc(kt), koff, 0, wave);
+    dma_half_tile_buf<4>(sVA, v_rsrc(kt), voff, 0, wave);
+  }
+
+  const int q_l = wave * 32 + l32;
+  const int qrow = qt * kTile + q_l;
   const bf16* qp = p.q + b * p.qs.b + (int64_t)qrow * p.qs.s + h * p.qs.h + hi * 8;
   const bf16* dop = p.dout + b * p.ds.b + (int64_t)qrow * p.ds.s + h * p.ds.h + hi * 8;
   bf16x8 qf[8], dof[8];
@@ -167,48 +312,27 @@ __global__ __launch_bounds__(256, 2) void dq_kernel(const BwdParams p) {
   f32x16 dq[4];
 #pragma unroll
   for (int i = 0; i < 4; ++i) dq[i] = f32x16{0};
-  const bf16* kbase = p.k + b * p.ks.b + h * p.ks.h;
-  const bf16* vbase = p.v + b * p.vs.b + h * p.vs.h;
   const TrLane tr(lane);
-  const int q_l = wave * 32 + l32;
 
-  const int e0 = p.ptr[qt], e1 = p.ptr[qt + 1];
   for (int e = e0; e < e1; ++e) {
-    const int kt = p.idx[e];
-    const int causal = p.flag[e];
-    if ((unsigned)kt >= (unsigned)p.n_ktiles) continue;
-    __syncthreads();
-    stage_tile<lds_off_u>(sK, kbase + (int64_t)kt * kTile * p.ks.s, p.ks.s, tid);
-    stage_tile<lds_off_k>(sV, vbase + (int64_t)kt * kTile * p.vs.s, p.vs.s, tid);
-    __syncthreads();
-
-#pragma unroll 1
-    for (int mb = 0; mb < 4; ++mb) {     // 32 keys at a time
-      f32x16 s = f32x16{0}, dp = f32x16{0};
-#pragma unroll
-      for (int ks = 0; ks < 8; ++ks) {
-        const bf16x8 ak = lds_read_b128(sK, lds_off_u(32 * mb + l32, 2 * ks + hi));
-        s = mfma32(ak, qf[ks], s);
-        const bf16x8 av = lds_read_b128(sV, lds_off_k(32 * mb + l32, 2 * ks + hi));
-        dp = mfma32(av, dof[ks], dp);
-      }
-      // element i: key 32*mb + 8*(i/4) + 4*hi + i%4, query column q_l
-      bf16x8 dsb[2];
-#pragma unroll
-      for (int i = 0; i < 16; ++i) {
-        const int key = 32 * mb + 8 * (i >> 2) + 4 * hi + (i & 3);
-        float pv = fast_exp2(fmaf(s[i], p.scale_log2, -lse2));
-        if (causal && key > q_l) pv = 0.f;
-        dsb[i >> 3][i & 7] = (bf16)(pv * (dp[i] - delta));
-      }
-#pragma unroll
-      for (int t = 0; t < 2; ++t)
-#pragma unroll
-        for (int mbd = 0; mbd < 4; ++mbd) {
-          const bf16x8 a_k = lds_read_tr_frag<lds_off_u>(sK, tr, 32 * mb + 16 * t, mbd);
-          dq[mbd] = mfma32(a_k, dsb[t], dq[mbd]);
-        }
+    const int causal = sload(p.flag, e);
+    const int kt_next = e + 1 < e1 ? ktile(e + 1) : kt;
+    wait_vmem_all();
+    __syncthreads();            // stage A (keys 0..63) landed; everyone is done with stage B
+    dma_half_tile_buf<4>(sKB, k_rsrc(kt), koff, k_half, wave);
+    dma_half_tile_buf<4>(sVB, v_rsrc(kt), voff, v_half, wave);
+    // causal tile: queries 64..127 (waves 2, 3) see all of keys 0..63
+    dq_half_tile(sKA, sVA, qf, dof, dq, tr, p.scale_log2, lse2, delta, l32, hi, q_l, 0, causal && wave < 2);
+    wait_vmem_all();
+    __syncthreads();            // stage B landed; everyone is done with stage A
+    if (e + 1 < e1) {
+      dma_half_tile_buf<4>(sKA, k_rsrc(kt_next), koff, 0, wave);
+      dma_half_tile_buf<4>(sVA, v_rsrc(kt_next), voff, 0, wave);
     }
+    // causal tile: queries 0..63 (waves 0, 1) see none of keys 64..127
+    if (!causal || wave >= 2)
+      dq_half_tile(sKB, sVB, qf, dof, dq, tr, p.scale_log2, lse2, delta, l32, hi, q_l, kHalf, causal);
+    kt = kt_next;
   }
   store_acc_t(p.out0 + b * p.o0s.b + (int64_t)qrow * p.o0s.s + h * p.o0s.h, dq, p.scale, hi);
 }
@@ -224,6 +348,8 @@ static int fill_common(BwdParams& p, const void* q, const void* k, const void* v
   if (head_dim != kHeadDim || !(softmax_scale > 0.f)) return UA_ERR_UNSUPPORTED;
   if (!aligned16(q) || !aligned16(k) || !aligned16(v) || !aligned16(dout)) return UA_ERR_ALIGN;
   if (!strides_ok(qs) || !strides_ok(ks) || !strides_ok(vs) || !strides_ok(ds)) return UA_ERR_ALIGN;
+  for (const int64_t* st : {qs, ks, vs, ds})
+    if (st[1] > (INT32_MAX >> 9)) return UA_ERR_SHAPE;
   p.q = (const bf16*)q; p.k = (const bf16*)k; p.v = (const bf16*)v; p.dout = (const bf16*)dout;
   p.lse = lse; p.delta = delta;
   p.batch = batch; p.n_heads = n_heads; p.n_qtiles = n_qtiles; p.n_ktiles = n_ktiles;

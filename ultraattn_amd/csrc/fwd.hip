@@ -126,12 +126,12 @@ __global__ __launch_bounds__(256, 2) void fwd_kernel(const FwdParams p) {
   const int l32 = lane & 31, hi = lane >> 5;
   int pos, bh;
   map_block(blockIdx.x, p.batch * p.n_heads, p.heads_per_xcd, pos, bh);
-  const int qt = p.q_order[pos];
+  const int qt = sload(p.q_order, pos);
   const int b = bh / p.n_heads, h = bh % p.n_heads;
 
   const bf16* kbase = p.k + b * p.ks.b + h * p.ks.h;
   const bf16* vbase = p.v + b * p.vs.b + h * p.vs.h;
-  const int e0 = p.row_ptr[qt], e1 = p.row_ptr[qt + 1];
+  const int e0 = sload(p.row_ptr, qt), e1 = sload(p.row_ptr, qt + 1);
   const int k_stride = (int)p.ks.s, v_stride = (int)p.vs.s;
   int koff[4], voff[4];
   dma_voffsets<lds_off_k, 4>(koff, k_stride, wave, lane);
@@ -143,7 +143,7 @@ __global__ __launch_bounds__(256, 2) void fwd_kernel(const FwdParams p) {
   auto v_rsrc = [&](int kt) { return make_rsrc(vbase + (int64_t)kt * kTile * v_stride, v_extent); };
 
   // first half tile of the first entry goes in flight before anything else
-  int kt = e0 < e1 ? min(max(p.col_idx[e0], 0), p.n_ktiles - 1) : 0;
+  int kt = e0 < e1 ? min(max(sload(p.col_idx, e0), 0), p.n_ktiles - 1) : 0;
   if (e0 < e1) {
     dma_half_tile_buf<4>(sKA, k_rsrc(kt), koff, 0, wave);
     dma_half_tile_buf<4>(sVA, v_rsrc(kt), voff, 0, wave);
@@ -165,8 +165,8 @@ __global__ __launch_bounds__(256, 2) void fwd_kernel(const FwdParams p) {
   const TrLane tr(lane);
 
   for (int e = e0; e < e1; ++e) {
-    const int causal = p.flag[e];
-    const int kt_next = e + 1 < e1 ? min(max(p.col_idx[e + 1], 0), p.n_ktiles - 1) : kt;
+    const int causal = sload(p.flag, e);
+    const int kt_next = e + 1 < e1 ? min(max(sload(p.col_idx, e + 1), 0), p.n_ktiles - 1) : kt;
     // stage A (keys 0..63 of this tile) has landed; everyone is done with stage B
     wait_vmem_all();
     __syncthreads();

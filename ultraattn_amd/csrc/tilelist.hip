@@ -18,6 +18,27 @@ __host__ __device__ __forceinline__ int tile_type(const uint8_t* mask, int nkb, 
   return a == b ? 2 : (a > b ? 1 : 0);
 }
 
+// Launch order: does row a come before row b?  Rows much longer than average
+// (len * n > 2 * nnz) first, longest first; the rest in lexicographic order of their index
+// lists, a list that is a prefix of another sorting after it; ties by row number.  Rows that
+// walk the same K/V (or Q/dO) tiles thus sit next to each other in the launch.
+__host__ __device__ __forceinline__ bool row_precedes(const int32_t* ptr, const int32_t* idx, int n, int a, int b) {
+  const int pa = ptr[a], pb = ptr[b];
+  const int la = ptr[a + 1] - pa, lb = ptr[b + 1] - pb;
+  const int64_t nnz2 = 2 * (int64_t)ptr[n];
+  const bool va = (int64_t)la * n > nnz2, vb = (int64_t)lb * n > nnz2;
+  if (va != vb) return va;
+  if (!va) {
+    const int m = la < lb ? la : lb;
+    for (int t = 0; t < m; ++t) {
+      const int ca = idx[pa + t], cb = idx[pb + t];
+      if (ca != cb) return ca < cb;
+    }
+  }
+  if (la != lb) return la > lb;
+  return a < b;
+}
+
 static int check_mask(const uint8_t* mask, int nqb, int nkb, int rate) {
   if (!mask) return UA_ERR_NULL;
   if (nqb <= 0 || nkb <= 0 || rate <= 0) return UA_ERR_SHAPE;
@@ -44,9 +65,8 @@ __global__ void tl_count_kernel(const uint8_t* mask, int nqb, int nkb, int rate,
   }
 }
 
-// scan + order: a single workgroup turns counts into exclusive prefix sums and computes the
-// longest-first stable rank of every row by counting (rank = #rows that must come earlier).
-__global__ __launch_bounds__(1024) void tl_scan_kernel(const int32_t* cnt, int n, int32_t* ptr, int32_t* order) {
+// scan: a single workgroup turns counts into exclusive prefix sums.
+__global__ __launch_bounds__(1024) void tl_scan_kernel(const int32_t* cnt, int n, int32_t* ptr) {
   __shared__ int32_t part[1024];
   const int tid = threadIdx.x;
   const int per = (n + 1023) / 1024;
@@ -64,15 +84,21 @@ __global__ __launch_bounds__(1024) void tl_scan_kernel(const int32_t* cnt, int n
   int run = tid ? part[tid - 1] : 0;
   for (int i = lo; i < hi; ++i) { ptr[i] = run; run += cnt[i]; }
   if (tid == 1023) ptr[n] = part[1023];
-  for (int i = tid; i < n; i += 1024) {
-    const int ci = cnt[i];
-    int rank = 0;
-    for (int j = 0; j < n; ++j) {
-      const int cj = cnt[j];
-      rank += (cj > ci) || (cj == ci && j < i);
-    }
-    order[rank] = i;
-  }
+}
+
+// order: rank of a row = number of rows that precede it (one thread per row).
+__global__ void tl_order_kernel(const int32_t* qptr, const int32_t* qidx, int nq, int32_t* q_order,
+                                const int32_t* kptr, const int32_t* kidx, int nk, int32_t* k_order) {
+  const int t = blockIdx.x * blockDim.x + threadIdx.x;
+  const int32_t* ptr = t < nq ? qptr : kptr;
+  const int32_t* idx = t < nq ? qidx : kidx;
+  const int n = t < nq ? nq : nk;
+  int32_t* order = t < nq ? q_order : k_order;
+  const int i = t < nq ? t : t - nq;
+  if (t >= nq + nk) return;
+  int rank = 0;
+  for (int j = 0; j < n; ++j) rank += (j != i) && row_precedes(ptr, idx, n, j, i);
+  order[rank] = i;
 }
 
 __global__ void tl_fill_kernel(const uint8_t* mask, int nqb, int nkb, int rate,
@@ -148,10 +174,9 @@ extern "C" int ua_tilelist_build(const uint8_t* block_mask, int n_qblocks, int n
       row_idx[pos] = qt; cflag[pos] = flag[i];
     }
   std::iota(q_order, q_order + nqt, 0);
-  std::stable_sort(q_order, q_order + nqt, [&](int32_t a, int32_t b) {
-    return row_ptr[a + 1] - row_ptr[a] > row_ptr[b + 1] - row_ptr[b]; });
+  std::sort(q_order, q_order + nqt, [&](int32_t a, int32_t b) { return row_precedes(row_ptr, col_idx, nqt, a, b); });
   std::iota(k_order, k_order + nkt, 0);
-  std::stable_sort(k_order, k_order + nkt, [&](int32_t a, int32_t b) { return kcnt[a] > kcnt[b]; });
+  std::sort(k_order, k_order + nkt, [&](int32_t a, int32_t b) { return row_precedes(col_ptr, row_idx, nkt, a, b); });
   return UA_OK;
 }
 
@@ -171,9 +196,12 @@ extern "C" int ua_tilelist_build_device(const uint8_t* block_mask, int n_qblocks
   int32_t* kcnt = work + nqt + 1;
   const int blocks = (nqt + nkt + 255) / 256;
   hipLaunchKernelGGL(tl_count_kernel, dim3(blocks), dim3(256), 0, st, block_mask, n_qblocks, n_kblocks, rate, qcnt, kcnt);
-  hipLaunchKernelGGL(tl_scan_kernel, dim3(1), dim3(1024), 0, st, (const int32_t*)qcnt, nqt, row_ptr, q_order);
-  hipLaunchKernelGGL(tl_scan_kernel, dim3(1), dim3(1024), 0, st, (const int32_t*)kcnt, nkt, col_ptr, k_order);
+  hipLaunchKernelGGL(tl_scan_kernel, dim3(1), dim3(1024), 0, st, (const int32_t*)qcnt, nqt, row_ptr);
+  hipLaunchKernelGGL(tl_scan_kernel, dim3(1), dim3(1024), 0, st, (const int32_t*)kcnt, nkt, col_ptr);
   hipLaunchKernelGGL(tl_fill_kernel, dim3(blocks), dim3(256), 0, st, block_mask, n_qblocks, n_kblocks, rate,
                      (const int32_t*)row_ptr, col_idx, flag, (const int32_t*)col_ptr, row_idx, cflag);
+  hipLaunchKernelGGL(tl_order_kernel, dim3((nqt + nkt + 63) / 64), dim3(64), 0, st,
+                     (const int32_t*)row_ptr, (const int32_t*)col_idx, nqt, q_order,
+                     (const int32_t*)col_ptr, (const int32_t*)row_idx, nkt, k_order);
   return hipGetLastError() == hipSuccess ? UA_OK : UA_ERR_LAUNCH;
 }

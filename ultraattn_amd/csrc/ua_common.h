@@ -129,6 +129,17 @@ __device__ __forceinline__ void dma_half_tile(unsigned char* lds, const bf16* g,
   for (int i = 0; i < 16 / NW; ++i) dma16(g + off[i], lds + (NW * i + wave) * 1024);
 }
 
+// Wave-uniform reads of the (read-only) tile-list arrays through the scalar cache.
+__device__ __forceinline__ int32_t sload(const int32_t* p, int i) {
+  return ((const __attribute__((address_space(4))) int32_t*)p)[i];
+}
+__device__ __forceinline__ int sload(const uint8_t* p, int i) {
+  // the scalar unit loads dwords: fetch the aligned word that holds byte i
+  const uintptr_t a = reinterpret_cast<uintptr_t>(p) + (uintptr_t)i;
+  const uint32_t w = *reinterpret_cast<const __attribute__((address_space(4))) uint32_t*>(a & ~(uintptr_t)3);
+  return (w >> (8 * (a & 3))) & 0xff;
+}
+
 // Buffer-addressed variant (buffer_load_dwordx4 ... lds): the source address is
 // descriptor base + per-lane byte offset `voff` + wave-uniform byte offset `soff`, so a tile's
 // address arithmetic stays on the scalar unit; reads beyond the descriptor's extent return 0.
@@ -137,6 +148,9 @@ __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* base, ui
 }
 __device__ __forceinline__ void dma16_buf(__amdgpu_buffer_rsrc_t r, unsigned char* lds_dst, int voff, int soff) {
   __builtin_amdgcn_raw_ptr_buffer_load_lds(r, (__attribute__((address_space(3))) void*)lds_dst, 16, voff, soff, 0, 0);
+}
+__device__ __forceinline__ void dma4_buf(__amdgpu_buffer_rsrc_t r, unsigned char* lds_dst, int voff, int soff) {
+  __builtin_amdgcn_raw_ptr_buffer_load_lds(r, (__attribute__((address_space(3))) void*)lds_dst, 4, voff, soff, 0, 0);
 }
 // Per-thread byte offsets for staging a [64][128] bf16 half tile with NW waves (see dma_offsets).
 template <int (*OFF)(int, int), int NW>

@@ -18,7 +18,7 @@ _HOST_FIELDS = ("row_ptr", "col_idx", "flag", "col_ptr", "row_idx", "cflag", "q_
 @dataclass
 class TileList:
     """CSR over query tiles (``row_ptr, col_idx, flag``), CSC over key tiles
-    (``col_ptr, row_idx, cflag``) and the longest-first launch orders, as host numpy arrays;
+    (``col_ptr, row_idx, cflag``) and the launch orders (rows that share tiles adjacent, very long rows first), as host numpy arrays;
     ``on(device)`` gives (and caches) device copies."""
     n_qtiles: int
     n_ktiles: int
