@@ -25,6 +25,11 @@ HBM_PEAK_GBPS = 8000.0            # MI355X HBM3E, published
 FLOP_PER_CLK_PER_CU = 4096        # dense bf16 MFMA, CDNA4
 
 
+# HBM bytes per launch of the dominant kernel, from profiles/hbm_traffic_<workload>.txt
+# (rocprofv3 --pmc FETCH_SIZE x 2.0 + WRITE_SIZE x 1.0, scaling explained there).
+TRAFFIC_BYTES = {("c3", "dkdv_kernel"): 43.52e9, ("c5", "fwd_kernel"): 12.37e9}
+
+
 def log(*a):
     print(*a, file=sys.stderr, flush=True)
 
@@ -209,6 +214,34 @@ def run_c5(steps, warmup):
             "fwd_plus_merge_tflops": F / wall_ms / 1e9}
 
 
+def probe_mfma(peak):
+    """Sustained register-only MFMA rate with constant and with random operand bits."""
+    import torch
+    from ultraattn_amd import _lib
+    lib = _lib.load()
+    dev = "cuda:0"
+    n_blocks, iters = 512, 40000
+    out = torch.empty(n_blocks * 256, dtype=torch.float32, device=dev)
+    g = torch.Generator(device=dev).manual_seed(0)
+    ops_ = {"constant": torch.ones(512 * 8, dtype=torch.bfloat16, device=dev),
+            "random": torch.randn(512 * 8, dtype=torch.float32, device=dev, generator=g).to(torch.bfloat16)}
+    res = {}
+    st = torch.cuda.current_stream().cuda_stream
+    for name, t in ops_.items():
+        _lib.check(lib.ua_probe_mfma(t.data_ptr(), out.data_ptr(), n_blocks, 2000, st), "ua_probe_mfma")
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        _lib.check(lib.ua_probe_mfma(t.data_ptr(), out.data_ptr(), n_blocks, iters, st), "ua_probe_mfma")
+        e1.record()
+        torch.cuda.synchronize()
+        ms = e0.elapsed_time(e1)
+        res[name + "_operands_tflops"] = n_blocks * 4 * 4 * iters * 32768.0 / ms / 1e9
+    res["note"] = ("register-only v_mfma_f32_32x32x16_bf16 loop, 2 waves per SIMD; the clock follows power, "
+                   "power follows operand bit activity")
+    return res
+
+
 def cpu_baseline():
     """The reference's block-loop path restated on the CPU (oracle.block_loop_fwd), timed on
     config 1 exactly: B=1, S=8192, Nh=8, d=128, fp32, 16x16 causal block grid, forward only."""
@@ -242,6 +275,8 @@ def main():
     ap.add_argument("--workload", default="c3", choices=["c2", "c3", "c4", "c5"])
     ap.add_argument("--no-extra", action="store_true", help="skip the other workloads")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also run one plain 1 GiB device copy (known size, for scaling rocprof byte counters)")
     a = ap.parse_args()
     if a.gpus != 1:
         sys.exit("bench.py measures one GPU's share of the path: run it with --gpus 1 "
@@ -254,6 +289,12 @@ def main():
     peak = prop.multi_processor_count * FLOP_PER_CLK_PER_CU * clock_ghz / 1e3      # TFLOP/s
     log(f"device {prop.name}: {prop.multi_processor_count} CUs @ {clock_ghz:.2f} GHz -> bf16 MFMA peak {peak:.1f} TFLOP/s")
 
+    if a.calibrate_copy:
+        src = torch.empty(1 << 30, dtype=torch.uint8, device="cuda:0")
+        dst = torch.empty_like(src)
+        dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
     if a.workload == "c5":
         main_res = run_c5(a.steps, a.warmup)
     else:
@@ -265,15 +306,17 @@ def main():
         F = main_res["fwd_flops"]
         # dominant kernel: dK/dV.  Algorithmic flops of that launch: 4 of the backward's 5 GEMMs.
         roof = {"kernel": "dkdv_kernel", "bound": "mfma", "achieved": 2.0 * F / kt["dkdv"] / 1e9, "peak": peak,
-                "unit": "TFLOP/s", "traffic": None, "kernel_ms": kt["dkdv"]}
+                "unit": "TFLOP/s", "traffic": TRAFFIC_BYTES.get((a.workload, "dkdv_kernel")), "kernel_ms": kt["dkdv"],
+                "algorithmic_flops": 2.0 * F}
         main_res.update(dkdv_ms=kt["dkdv"], dq_ms=kt["dq"], dkdv_tflops=2.0 * F / kt["dkdv"] / 1e9,
                         dq_tflops=0.5 * F / kt["dq"] / 1e9)
         value = main_res["fwd_bwd_tflops"]
         metric = "effective TFLOP/s on active blocks, forward+backward"
     else:
-        ms = main_res["fwd_ms"]
+        launches = 4 if a.workload == "c5" else 1          # c5 runs the forward as 4 kernel tiles
         roof = {"kernel": "fwd_kernel", "bound": "mfma", "achieved": main_res["fwd_tflops"], "peak": peak,
-                "unit": "TFLOP/s", "traffic": None, "kernel_ms": ms}
+                "unit": "TFLOP/s", "traffic": TRAFFIC_BYTES.get((a.workload, "fwd_kernel")),
+                "kernel_ms": main_res["fwd_ms"] / launches, "algorithmic_flops": main_res["fwd_flops"] / launches}
         value = main_res.get("fwd_plus_merge_tflops", main_res["fwd_tflops"])
         metric = "effective TFLOP/s on active blocks, forward"
     roof["frac"] = roof["achieved"] / roof["peak"]
@@ -304,6 +347,8 @@ def main():
                       "seq_kv": int(workload_mask(a.workload).shape[1]) * BLOCK},
            "frac_of_bf16_mfma_peak": value / peak, "peak_tflops": peak, "detail": main_res,
            "fwd_frac_of_peak": main_res["fwd_tflops"] / peak, "roofline": roof, "extra": extra}
+    out["mfma_probe"] = probe_mfma(peak)
+    log(json.dumps(out["mfma_probe"]))
     if not a.no_cpu:
         out["cpu_baseline"] = cpu_baseline()
         log(json.dumps(out["cpu_baseline"]))

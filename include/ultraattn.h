@@ -130,6 +130,14 @@ int ua_bsa_bwd_dq(const void *q, const void *k, const void *v, const void *dout,
 int ua_merge(const void *const *o_parts, const float *const *lse_parts, int n_parts,
              void *o, float *lse, int batch, int seqlen, int n_heads, int head_dim, void *stream);
 
+/* ---- diagnostic (no counterpart in the reference) ----------------------------------------------
+ * Runs n_blocks workgroups of 256 threads, each wave issuing 4 * iters register-only
+ * v_mfma_f32_32x32x16_bf16 (32768 flop each) on the 512 x 16 bytes of operand bits at `operands`
+ * (device, 16-byte aligned); `out` receives n_blocks * 256 floats.  Timed by the caller, it gives
+ * the matrix pipe's sustained rate for those operand bits: the benchmark reports it beside the
+ * attention kernels because the part's clock follows the power its operands make it draw.     */
+int ua_probe_mfma(const void *operands, float *out, int n_blocks, int iters, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

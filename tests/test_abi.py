@@ -23,7 +23,7 @@ def test_header_symbols_are_exported(lib):
     names = declared_symbols()
     assert {"ua_bsa_fwd", "ua_bsa_bwd_dkdv", "ua_bsa_bwd_dq", "ua_bsa_bwd_delta", "ua_merge",
             "ua_tilelist_build", "ua_tilelist_size", "ua_tilelist_build_device", "ua_strerror",
-            "ua_version"} <= set(names)
+            "ua_version", "ua_probe_mfma"} <= set(names)
     raw = ctypes.CDLL(LIB_PATH)
     for n in names:
         assert hasattr(raw, n), f"{n} declared in include/ultraattn.h but not exported"

@@ -29,6 +29,27 @@ __global__ __launch_bounds__(256) void merge_kernel(const MergeParams p) {
   const int ntok = min(kTok, p.seqlen - s0);       // the last workgroup of a batch may be ragged
   const int rows = ntok * p.n_heads;
 
+  // The rows are streamed as 16-byte chunks (chunk c = 8 bf16 of row c/16), kUnroll chunks per
+  // thread per step, and the loads of step n+1 are issued before step n is combined, so that
+  // P * kUnroll (..2x) 16-byte loads per thread are always in flight.
+  const int64_t base = ((int64_t)b * p.seqlen + s0) * p.n_heads * kHeadDim;
+  const int n_chunks = rows * 16;
+  constexpr int kUnroll = P <= 4 ? 4 : (P <= 8 ? 2 : 1);
+  constexpr int kStep = 256 * kUnroll;
+  u32x4 raw[kUnroll][P];
+  auto load = [&](int c0) {
+#pragma unroll
+    for (int u = 0; u < kUnroll; ++u) {
+      const int c = c0 + u * 256;
+      if (c < n_chunks) {
+#pragma unroll
+        for (int i = 0; i < P; ++i)
+          raw[u][i] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p.o_parts[i] + base) + c);
+      }
+    }
+  };
+  load(tid);        // first step's rows are in flight while the statistics are handled
+
   // phase 1: one thread per (head, token): statistics, coalesced along the token axis
   for (int t = tid; t < kTok * p.n_heads; t += 256) {
     const int h = t / kTok, sl = t % kTok;
@@ -50,31 +71,36 @@ __global__ __launch_bounds__(256) void merge_kernel(const MergeParams p) {
   }
   __syncthreads();
 
-  // phase 2: stream the rows; chunk c covers 8 bf16 of row c/16
-  const int64_t base = ((int64_t)b * p.seqlen + s0) * p.n_heads * kHeadDim;
-  const int n_chunks = rows * 16;
-  for (int c = tid; c < n_chunks; c += 256) {
-    const int row = c >> 4;
-    u32x4 raw[P];
+  // phase 2: combine
+  for (int c0 = tid; c0 < n_chunks; c0 += kStep) {
+    u32x4 cur[kUnroll][P];
 #pragma unroll
-    for (int i = 0; i < P; ++i)
-      raw[i] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p.o_parts[i] + base) + c);
-    float acc[8];
+    for (int u = 0; u < kUnroll; ++u)
 #pragma unroll
-    for (int j = 0; j < 8; ++j) acc[j] = 0.f;
+      for (int i = 0; i < P; ++i) cur[u][i] = raw[u][i];
+    load(c0 + kStep);
 #pragma unroll
-    for (int i = 0; i < P; ++i) {
-      const float w = w_lds[i * rows + row];
+    for (int u = 0; u < kUnroll; ++u) {
+      const int c = c0 + u * 256;
+      if (c >= n_chunks) break;
+      const int row = c >> 4;
+      float acc[8];
 #pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        acc[2 * j] = fmaf(w, __uint_as_float(raw[i][j] << 16), acc[2 * j]);
-        acc[2 * j + 1] = fmaf(w, __uint_as_float(raw[i][j] & 0xffff0000u), acc[2 * j + 1]);
+      for (int j = 0; j < 8; ++j) acc[j] = 0.f;
+#pragma unroll
+      for (int i = 0; i < P; ++i) {
+        const float w = w_lds[i * rows + row];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          acc[2 * j] = fmaf(w, __uint_as_float(cur[u][i][j] << 16), acc[2 * j]);
+          acc[2 * j + 1] = fmaf(w, __uint_as_float(cur[u][i][j] & 0xffff0000u), acc[2 * j + 1]);
+        }
       }
-    }
-    bf16x8 out;
+      bf16x8 out;
 #pragma unroll
-    for (int j = 0; j < 8; ++j) out[j] = (bf16)acc[j];
-    __builtin_nontemporal_store(out, reinterpret_cast<bf16x8*>(p.o + base) + c);
+      for (int j = 0; j < 8; ++j) out[j] = (bf16)acc[j];
+      __builtin_nontemporal_store(out, reinterpret_cast<bf16x8*>(p.o + base) + c);
+    }
   }
 }
 
