@@ -75,72 +75,119 @@ __device__ __forceinline__ bf16x8 read_tr_pair(const unsigned char* smem, int of
   return __builtin_shufflevector(a, b, 0, 1, 2, 3, 4, 5, 6, 7);
 }
 
-// dK/dV: per query tile of the column, for each block of 32 query rows.
-__device__ __forceinline__ void dkdv_tile(const unsigned char* sQ, const unsigned char* sdO, const float* sLse,
-                                          const float* sDelta, const bf16x8 (&kf)[8], const bf16x8 (&vf)[8],
-                                          f32x16 (&dk)[4], f32x16 (&dv)[4], const LaneOffsU& lo, float scale_log2,
-                                          int hi, int key_l, bool causal) {
+// ---- dK/dV ------------------------------------------------------------------------------------
+// The workgroup has 8 wavefronts in two groups of 4; wave w of either group owns key rows
+// 32w..32w+31 of the key tile, and each SIMD hosts one wave of each group.  Per block of 32
+// query rows:
+//   group A:  S = Q K^T -> P = exp2(..) -> hands P (bf16) to its partner through LDS;  dV^T += dO^T P
+//   group B:  dP = dO V^T;  takes P;  dS = P * (dP - delta);                             dK^T += Q^T dS
+// Both groups issue 16 MFMAs per block and about the same vector work, fit in 256 registers
+// (two waves per SIMD, accumulators in VGPRs), and one group's MFMAs overlap the other's exp2 /
+// pointwise work.
+constexpr int kPBlockBytes = 4 * 2048;      // P of one 32-row block: 4 waves x (64 lanes x 32 B)
+
+__device__ __forceinline__ void dkdv_tile_a(const unsigned char* sQ, const unsigned char* sdO, const float* sLse,
+                                            unsigned char* sP, int& pbuf, const bf16x8 (&kf)[8], f32x16 (&dv)[4],
+                                            const LaneOffsU& lo, float scale_log2, int lane, int hi, int wave,
+                                            int key_l, bool causal) {
 #pragma unroll 1
   for (int nb = 0; nb < 4; ++nb) {     // 32 query rows at a time
-    // this block's per-lane offsets: 16 adds; everything else is an immediate offset
     const int blk = nb * 32 * kRowBytes;
     int nat[8], trb[4][2];
 #pragma unroll
     for (int ks = 0; ks < 8; ++ks) nat[ks] = lo.nat[ks] + blk;
 #pragma unroll
     for (int mbd = 0; mbd < 4; ++mbd) { trb[mbd][0] = lo.tr[mbd][0] + blk; trb[mbd][1] = lo.tr[mbd][1] + blk; }
-    f32x16 s = f32x16{0}, dp = f32x16{0};
+    f32x16 s = f32x16{0};
 #pragma unroll
-    for (int ks = 0; ks < 8; ++ks) {
-      const bf16x8 aq = lds_read_b128(sQ, nat[ks]);
-      s = mfma32(aq, kf[ks], s);
-      const bf16x8 ad = lds_read_b128(sdO, nat[ks]);
-      dp = mfma32(ad, vf[ks], dp);
-    }
+    for (int ks = 0; ks < 8; ++ks) s = mfma32(lds_read_b128(sQ, nat[ks]), kf[ks], s);
     // element i: query row 32*nb + 8*(i/4) + 4*hi + i%4, key column key_l
     if (causal) {
 #pragma unroll
       for (int i = 0; i < 16; ++i)
         if (key_l > 32 * nb + 8 * (i >> 2) + 4 * hi + (i & 3)) s[i] = -INFINITY;
     }
-    bf16x8 pb[2], dsb[2];
+    bf16x8 pb[2];
 #pragma unroll
     for (int g = 0; g < 4; ++g) {
-      const int q0 = 32 * nb + 8 * g + 4 * hi;
-      const f32x4 l4 = *reinterpret_cast<const f32x4*>(sLse + q0);
-      const f32x4 d4 = *reinterpret_cast<const f32x4*>(sDelta + q0);
+      const f32x4 l4 = *reinterpret_cast<const f32x4*>(sLse + 32 * nb + 8 * g + 4 * hi);
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
         const int i = 4 * g + j;
-        const float pv = fast_exp2(fmaf(s[i], scale_log2, -l4[j]));
-        const float dsv = pv * (dp[i] - d4[j]);
-        pb[i >> 3][i & 7] = (bf16)pv;
-        dsb[i >> 3][i & 7] = (bf16)dsv;
+        pb[i >> 3][i & 7] = (bf16)fast_exp2(fmaf(s[i], scale_log2, -l4[j]));
       }
     }
+    unsigned char* dst = sP + pbuf * kPBlockBytes + wave * 2048 + lane * 16;
+    *reinterpret_cast<bf16x8*>(dst) = pb[0];
+    *reinterpret_cast<bf16x8*>(dst + 1024) = pb[1];
+    pbuf ^= 1;
+    __syncthreads();                   // P of this block is visible to the partner wave
 #pragma unroll
     for (int t = 0; t < 2; ++t)
 #pragma unroll
       for (int mbd = 0; mbd < 4; ++mbd) {
         const bf16x8 a_do = read_tr_pair(sdO + 16 * t * kRowBytes, trb[mbd][0], trb[mbd][1]);
         dv[mbd] = mfma32(a_do, pb[t], dv[mbd]);
+      }
+  }
+}
+
+__device__ __forceinline__ void dkdv_tile_b(const unsigned char* sQ, const unsigned char* sdO, const float* sDelta,
+                                            const unsigned char* sP, int& pbuf, const bf16x8 (&vf)[8], f32x16 (&dk)[4],
+                                            const LaneOffsU& lo, int lane, int hi, int wave) {
+#pragma unroll 1
+  for (int nb = 0; nb < 4; ++nb) {
+    const int blk = nb * 32 * kRowBytes;
+    int nat[8], trb[4][2];
+#pragma unroll
+    for (int ks = 0; ks < 8; ++ks) nat[ks] = lo.nat[ks] + blk;
+#pragma unroll
+    for (int mbd = 0; mbd < 4; ++mbd) { trb[mbd][0] = lo.tr[mbd][0] + blk; trb[mbd][1] = lo.tr[mbd][1] + blk; }
+    f32x16 dp = f32x16{0};
+#pragma unroll
+    for (int ks = 0; ks < 8; ++ks) dp = mfma32(lds_read_b128(sdO, nat[ks]), vf[ks], dp);
+    __syncthreads();                   // the partner's P of this block has been written
+    const unsigned char* src = sP + pbuf * kPBlockBytes + wave * 2048 + lane * 16;
+    pbuf ^= 1;
+    u32x4 praw[2];
+    praw[0] = *reinterpret_cast<const u32x4*>(src);
+    praw[1] = *reinterpret_cast<const u32x4*>(src + 1024);
+    bf16x8 dsb[2];
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+      const f32x4 d4 = *reinterpret_cast<const f32x4*>(sDelta + 32 * nb + 8 * g + 4 * hi);
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int i = 4 * g + j;
+        const uint32_t w = praw[i >> 3][(i & 7) >> 1];
+        const float pv = __uint_as_float((i & 1) ? (w & 0xffff0000u) : (w << 16));
+        dsb[i >> 3][i & 7] = (bf16)(pv * (dp[i] - d4[j]));
+      }
+    }
+#pragma unroll
+    for (int t = 0; t < 2; ++t)
+#pragma unroll
+      for (int mbd = 0; mbd < 4; ++mbd) {
         const bf16x8 a_q = read_tr_pair(sQ + 16 * t * kRowBytes, trb[mbd][0], trb[mbd][1]);
         dk[mbd] = mfma32(a_q, dsb[t], dk[mbd]);
       }
   }
 }
 
-__global__ __launch_bounds__(256, 1) void dkdv_kernel(const BwdParams p) {
+__global__ __launch_bounds__(512) void dkdv_kernel(const BwdParams p) {
   // two stages (Q tile, dO tile, the rows' lse and delta), distinct arrays per stage
   __shared__ __attribute__((aligned(1024))) unsigned char sQ0[kTileBytes];
   __shared__ __attribute__((aligned(1024))) unsigned char sdO0[kTileBytes];
   __shared__ __attribute__((aligned(1024))) unsigned char sQ1[kTileBytes];
   __shared__ __attribute__((aligned(1024))) unsigned char sdO1[kTileBytes];
+  __shared__ __attribute__((aligned(1024))) unsigned char sP[2 * kPBlockBytes];
   __shared__ __attribute__((aligned(16))) float sStat0[2 * kTile];
   __shared__ __attribute__((aligned(16))) float sStat1[2 * kTile];
 
   const int tid = threadIdx.x, lane = tid & 63;
-  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wave8 = __builtin_amdgcn_readfirstlane(tid >> 6);      // 0..7
+  const bool group_b = wave8 >= 4;
+  const int wave = wave8 & 3;
   const int l32 = lane & 31, hi = lane >> 5;
   int pos, bh;
   map_block(blockIdx.x, p.batch * p.n_heads, p.heads_per_xcd, pos, bh);
@@ -148,19 +195,17 @@ __global__ __launch_bounds__(256, 1) void dkdv_kernel(const BwdParams p) {
   const int b = bh / p.n_heads, h = bh % p.n_heads;
   const int64_t seq_q = (int64_t)p.n_qtiles * kTile;
 
-  // K, V fragments (B operands): lane holds key row 32*wave + lane%32, d = 16*ks + 8*hi .. +7
+  // group A keeps the K fragments, group B the V fragments (B operands): lane holds key row
+  // 32*wave + lane%32, d = 16*ks + 8*hi .. +7
   const int krow = kt * kTile + wave * 32 + l32;
-  const bf16* kp = p.k + b * p.ks.b + (int64_t)krow * p.ks.s + h * p.ks.h + hi * 8;
-  const bf16* vp = p.v + b * p.vs.b + (int64_t)krow * p.vs.s + h * p.vs.h + hi * 8;
-  bf16x8 kf[8], vf[8];
+  const bf16* fp = group_b ? p.v + b * p.vs.b + (int64_t)krow * p.vs.s + h * p.vs.h + hi * 8
+                           : p.k + b * p.ks.b + (int64_t)krow * p.ks.s + h * p.ks.h + hi * 8;
+  bf16x8 frag[8];
 #pragma unroll
-  for (int ks = 0; ks < 8; ++ks) {
-    kf[ks] = *reinterpret_cast<const bf16x8*>(kp + ks * 16);
-    vf[ks] = *reinterpret_cast<const bf16x8*>(vp + ks * 16);
-  }
-  f32x16 dk[4], dv[4];
+  for (int ks = 0; ks < 8; ++ks) frag[ks] = *reinterpret_cast<const bf16x8*>(fp + ks * 16);
+  f32x16 acc[4];       // group A: dV^T, group B: dK^T
 #pragma unroll
-  for (int i = 0; i < 4; ++i) { dk[i] = f32x16{0}; dv[i] = f32x16{0}; }
+  for (int i = 0; i < 4; ++i) acc[i] = f32x16{0};
 
   const bf16* qbase = p.q + b * p.qs.b + h * p.qs.h;
   const bf16* dobase = p.dout + b * p.ds.b + h * p.ds.h;
@@ -171,9 +216,9 @@ __global__ __launch_bounds__(256, 1) void dkdv_kernel(const BwdParams p) {
   const int key_l = wave * 32 + l32;
 
   const int q_stride = (int)p.qs.s, do_stride = (int)p.ds.s;
-  int qoff[4], dooff[4];
-  dma_voffsets<lds_off_u, 4>(qoff, q_stride, wave, lane);
-  dma_voffsets<lds_off_u, 4>(dooff, do_stride, wave, lane);
+  int qoff[2], dooff[2];
+  dma_voffsets<lds_off_u, 8>(qoff, q_stride, wave8, lane);
+  dma_voffsets<lds_off_u, 8>(dooff, do_stride, wave8, lane);
   const int q_half = kHalf * q_stride * 2, do_half = kHalf * do_stride * 2;
   const uint32_t q_extent = (uint32_t)((kTile - 1) * q_stride + kHeadDim) * 2;
   const uint32_t do_extent = (uint32_t)((kTile - 1) * do_stride + kHeadDim) * 2;
@@ -181,20 +226,34 @@ __global__ __launch_bounds__(256, 1) void dkdv_kernel(const BwdParams p) {
   // rows' statistics: threads 0..127 carry lse (pre-multiplied by log2 e; -inf -> +inf so that
   // rows without keys give P = 0), threads 128..255 carry delta
   auto load_stat = [&](int qt) {
-    const float x = tid < kTile ? lse_row[qt * kTile + tid] : delta_row[qt * kTile + tid - kTile];
-    return tid < kTile ? (x == -INFINITY ? INFINITY : x * kLog2e) : x;
+    float x = 0.f;
+    if (tid < 2 * kTile) {
+      x = tid < kTile ? lse_row[qt * kTile + tid] : delta_row[qt * kTile + tid - kTile];
+      if (tid < kTile) x = (x == -INFINITY) ? INFINITY : x * kLog2e;
+    }
+    return x;
   };
   auto stage = [&](int qt, unsigned char* sQ, unsigned char* sdO) {
-    dma_tile_buf(sQ, make_rsrc(qbase + (int64_t)qt * kTile * q_stride, q_extent), qoff, q_half, wave);
-    dma_tile_buf(sdO, make_rsrc(dobase + (int64_t)qt * kTile * do_stride, do_extent), dooff, do_half, wave);
+    const __amdgpu_buffer_rsrc_t rq = make_rsrc(qbase + (int64_t)qt * kTile * q_stride, q_extent);
+    const __amdgpu_buffer_rsrc_t rd = make_rsrc(dobase + (int64_t)qt * kTile * do_stride, do_extent);
+    dma_half_tile_buf<8>(sQ, rq, qoff, 0, wave8);
+    dma_half_tile_buf<8>(sQ + kHalfBytes, rq, qoff, q_half, wave8);
+    dma_half_tile_buf<8>(sdO, rd, dooff, 0, wave8);
+    dma_half_tile_buf<8>(sdO + kHalfBytes, rd, dooff, do_half, wave8);
+  };
+  auto tile = [&](const unsigned char* sQ, const unsigned char* sdO, const float* sStat, int& pbuf, bool causal) {
+    if (group_b) dkdv_tile_b(sQ, sdO, sStat + kTile, sP, pbuf, frag, acc, lo, lane, hi, wave);
+    else         dkdv_tile_a(sQ, sdO, sStat, sP, pbuf, frag, acc, lo, p.scale_log2, lane, hi, wave, key_l, causal);
   };
 
   const int e0 = sload(p.ptr, kt), e1 = sload(p.ptr, kt + 1);
   if (e0 < e1) {
     const int qt = qtile(e0);
-    sStat0[tid] = load_stat(qt);
+    const float st0 = load_stat(qt);
+    if (tid < 2 * kTile) sStat0[tid] = st0;
     stage(qt, sQ0, sdO0);
   }
+  int pbuf = 0;
   // entries are taken two at a time: even ones through stage 0, odd ones through stage 1
   for (int e = e0; e < e1; e += 2) {
     const bool has1 = e + 1 < e1, has2 = e + 2 < e1;
@@ -206,9 +265,9 @@ __global__ __launch_bounds__(256, 1) void dkdv_kernel(const BwdParams p) {
       stat = load_stat(qt);
       stage(qt, sQ1, sdO1);
     }
-    dkdv_tile(sQ0, sdO0, sStat0, sStat0 + kTile, kf, vf, dk, dv, lo, p.scale_log2, hi, key_l, sload(p.flag, e) != 0);
+    tile(sQ0, sdO0, sStat0, pbuf, sload(p.flag, e) != 0);
     if (!has1) break;
-    sStat1[tid] = stat;
+    if (tid < 2 * kTile) sStat1[tid] = stat;
     wait_vmem_all();
     __syncthreads();                       // stage 1 landed; everyone is done with stage 0
     if (has2) {
@@ -216,11 +275,11 @@ __global__ __launch_bounds__(256, 1) void dkdv_kernel(const BwdParams p) {
       stat = load_stat(qt);
       stage(qt, sQ0, sdO0);
     }
-    dkdv_tile(sQ1, sdO1, sStat1, sStat1 + kTile, kf, vf, dk, dv, lo, p.scale_log2, hi, key_l, sload(p.flag, e + 1) != 0);
-    if (has2) sStat0[tid] = stat;
+    tile(sQ1, sdO1, sStat1, pbuf, sload(p.flag, e + 1) != 0);
+    if (has2 && tid < 2 * kTile) sStat0[tid] = stat;
   }
-  store_acc_t(p.out0 + b * p.o0s.b + (int64_t)krow * p.o0s.s + h * p.o0s.h, dk, p.scale, hi);
-  store_acc_t(p.out1 + b * p.o1s.b + (int64_t)krow * p.o1s.s + h * p.o1s.h, dv, 1.f, hi);
+  if (group_b) store_acc_t(p.out0 + b * p.o0s.b + (int64_t)krow * p.o0s.s + h * p.o0s.h, acc, p.scale, hi);
+  else         store_acc_t(p.out1 + b * p.o1s.b + (int64_t)krow * p.o1s.s + h * p.o1s.h, acc, 1.f, hi);
 }
 
 // dQ: one 64-key half tile for this wave's 32 query rows.
@@ -381,7 +440,7 @@ extern "C" int ua_bsa_bwd_dkdv(const void* q, const void* k, const void* v, cons
   p.o0s = {dk_strides[0], dk_strides[1], dk_strides[2]};
   p.o1s = {dv_strides[0], dv_strides[1], dv_strides[2]};
   p.ptr = col_ptr; p.idx = row_idx; p.flag = cflag; p.order = k_order;
-  hipLaunchKernelGGL(dkdv_kernel, dim3((unsigned)(batch * n_heads * n_ktiles)), dim3(256), 0, (hipStream_t)stream, p);
+  hipLaunchKernelGGL(dkdv_kernel, dim3((unsigned)(batch * n_heads * n_ktiles)), dim3(512), 0, (hipStream_t)stream, p);
   return hipGetLastError() == hipSuccess ? UA_OK : UA_ERR_LAUNCH;
 }
 

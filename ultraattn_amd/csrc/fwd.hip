@@ -44,14 +44,26 @@ __device__ __forceinline__ void half_tile(const unsigned char* sK, const unsigne
                                           f32x16 (&oacc)[4], SoftmaxState& st, const TrLane& tr, float scale_log2,
                                           int l32, int hi, int q_local, int key0, bool mask, bool first) {
   // ---- S^T = K Q^T : 2 blocks of 32 keys x 32 queries ------------------------------------
+  // The 16 K fragments are fetched kAhead reads ahead of the MFMA that consumes them, so the
+  // LDS latency is covered by the preceding MFMAs instead of being paid before each one.
   f32x16 s[2];
+  s[0] = f32x16{0};
+  s[1] = f32x16{0};
+  {
+    constexpr int kAhead = 4;
+    bf16x8 kfr[16];
 #pragma unroll
-  for (int mb = 0; mb < 2; ++mb) {
-    s[mb] = f32x16{0};
+    for (int i = 0; i < kAhead; ++i) kfr[i] = lds_read_b128(sK, lds_off_k(32 * (i & 1) + l32, 2 * (i >> 1) + hi));
+    __builtin_amdgcn_sched_group_barrier(0x100, kAhead, 0);   // kAhead LDS reads up front
 #pragma unroll
-    for (int ks = 0; ks < 8; ++ks) {
-      const bf16x8 a = lds_read_b128(sK, lds_off_k(32 * mb + l32, 2 * ks + hi));
-      s[mb] = mfma32(a, qf[ks], s[mb]);
+    for (int i = 0; i < 16; ++i) {
+      if (i + kAhead < 16) {
+        const int j = i + kAhead;
+        kfr[j] = lds_read_b128(sK, lds_off_k(32 * (j & 1) + l32, 2 * (j >> 1) + hi));
+      }
+      s[i & 1] = mfma32(kfr[i], qf[i >> 1], s[i & 1]);
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);   // then 1 MFMA, 1 LDS read, ...
+      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
     }
   }
   // element (mb, i) of this lane: key key0 + 32*mb + 8*(i/4) + 4*hi + i%4, query q_local
@@ -62,6 +74,11 @@ __device__ __forceinline__ void half_tile(const unsigned char* sK, const unsigne
       for (int i = 0; i < 16; ++i)
         if (key0 + 32 * mb + 8 * (i >> 2) + 4 * hi + (i & 3) > q_local) s[mb][i] = -INFINITY;
   }
+  // the first V^T fragments are fetched now: their latency hides behind the softmax
+  constexpr int kVAhead = 3;
+  bf16x8 vfr[4];
+#pragma unroll
+  for (int i = 0; i < kVAhead; ++i) vfr[i] = lds_read_tr_frag<lds_off_v>(sV, tr, 16 * (i >> 2), i & 3);
   // ---- online softmax (fp32, log2 domain) ---------------------------------------------------
   float rs = 0.f;
   bf16x8 pf[4];
@@ -105,12 +122,12 @@ __device__ __forceinline__ void half_tile(const unsigned char* sK, const unsigne
   st.l_run += rs;
   // ---- O^T += V^T P^T : 4 blocks of 32 d x 32 queries, 4 steps of 16 keys -------------------
 #pragma unroll
-  for (int kk = 0; kk < 4; ++kk)
-#pragma unroll
-    for (int mbd = 0; mbd < 4; ++mbd) {
-      const bf16x8 a = lds_read_tr_frag<lds_off_v>(sV, tr, 16 * kk, mbd);
-      oacc[mbd] = mfma32(a, pf[kk], oacc[mbd]);
-    }
+  for (int i = 0; i < 16; ++i) {
+    if (i + kVAhead < 16) vfr[(i + kVAhead) & 3] = lds_read_tr_frag<lds_off_v>(sV, tr, 16 * ((i + kVAhead) >> 2), (i + kVAhead) & 3);
+    oacc[i & 3] = mfma32(vfr[i & 3], pf[i >> 2], oacc[i & 3]);
+    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);   // 1 MFMA
+    __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);   // 2 LDS reads (one fragment)
+  }
 }
 
 __global__ __launch_bounds__(256, 2) void fwd_kernel(const FwdParams p) {
