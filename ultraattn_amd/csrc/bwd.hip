@@ -86,69 +86,99 @@ __device__ __forceinline__ bf16x8 read_tr_pair(const unsigned char* smem, int of
 // pointwise work.
 constexpr int kPBlockBytes = 4 * 2048;      // P of one 32-row block: 4 waves x (64 lanes x 32 B)
 
+// Eight transposed fragments (2 steps of 16 rows x 4 d-blocks) feeding acc[mbd] += X^T * bfrag[t],
+// fetched kAhead fragments ahead of the MFMA that consumes them.
+__device__ __forceinline__ void mfma_tr_block(const unsigned char* sX, const LaneOffsU& lo, int blk,
+                                              const bf16x8 (&bfrag)[2], f32x16 (&acc)[4]) {
+  constexpr int kAhead = 3;
+  bf16x8 fr[8];
+#pragma unroll
+  for (int i = 0; i < kAhead; ++i)
+    fr[i] = read_tr_pair(sX + 16 * (i >> 2) * kRowBytes, lo.tr[i & 3][0] + blk, lo.tr[i & 3][1] + blk);
+  __builtin_amdgcn_sched_group_barrier(0x100, 2 * kAhead, 0);
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    if (i + kAhead < 8) {
+      const int j = i + kAhead;
+      fr[j] = read_tr_pair(sX + 16 * (j >> 2) * kRowBytes, lo.tr[j & 3][0] + blk, lo.tr[j & 3][1] + blk);
+    }
+    acc[i & 3] = mfma32(fr[i], bfrag[i >> 2], acc[i & 3]);
+    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+    __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+  }
+}
+
+// One 32x32 block X[rows 32*nb.., :] * frag^T over head_dim: the 8 row fragments are all fetched
+// before the dependent MFMA chain starts.
+__device__ __forceinline__ f32x16 mfma_nat_block(const unsigned char* sX, const LaneOffsU& lo, int blk,
+                                                 const bf16x8 (&frag)[8]) {
+  bf16x8 fr[8];
+#pragma unroll
+  for (int ks = 0; ks < 8; ++ks) fr[ks] = lds_read_b128(sX, lo.nat[ks] + blk);
+  __builtin_amdgcn_sched_group_barrier(0x100, 8, 0);
+  f32x16 acc = f32x16{0};
+#pragma unroll
+  for (int ks = 0; ks < 8; ++ks) acc = mfma32(fr[ks], frag[ks], acc);
+  return acc;
+}
+
+// S^T block -> P (bf16, accumulator layout) for query rows 32*nb.., written to the hand-over slot.
+__device__ __forceinline__ void dkdv_p_block(const unsigned char* sQ, const float* sLse, unsigned char* p_slot,
+                                             const bf16x8 (&kf)[8], const LaneOffsU& lo, float scale_log2, int nb,
+                                             int hi, int key_l, bool causal, bf16x8 (&pb)[2]) {
+  f32x16 s = mfma_nat_block(sQ, lo, nb * 32 * kRowBytes, kf);
+  // element i: query row 32*nb + 8*(i/4) + 4*hi + i%4, key column key_l
+  if (causal) {
+    keep_branch();
+#pragma unroll
+    for (int i = 0; i < 16; ++i)
+      if (key_l > 32 * nb + 8 * (i >> 2) + 4 * hi + (i & 3)) s[i] = -INFINITY;
+  }
+#pragma unroll
+  for (int g = 0; g < 4; ++g) {
+    const f32x4 l4 = *reinterpret_cast<const f32x4*>(sLse + 32 * nb + 8 * g + 4 * hi);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int i = 4 * g + j;
+      pb[i >> 3][i & 7] = (bf16)fast_exp2(fmaf(s[i], scale_log2, -l4[j]));
+    }
+  }
+  *reinterpret_cast<bf16x8*>(p_slot) = pb[0];
+  *reinterpret_cast<bf16x8*>(p_slot + 1024) = pb[1];
+}
+
+// Group A runs one block ahead of its partner: P of block nb+1 is produced before the
+// workgroup barrier of block nb, so its exp2 work overlaps the partner's MFMAs.  Three hand-over
+// slots: P(nb+2) may be written while the partner still reads P(nb).
 __device__ __forceinline__ void dkdv_tile_a(const unsigned char* sQ, const unsigned char* sdO, const float* sLse,
-                                            unsigned char* sP, int& pbuf, const bf16x8 (&kf)[8], f32x16 (&dv)[4],
+                                            unsigned char* sP, int& pslot, const bf16x8 (&kf)[8], f32x16 (&dv)[4],
                                             const LaneOffsU& lo, float scale_log2, int lane, int hi, int wave,
                                             int key_l, bool causal) {
+  unsigned char* mine = sP + wave * 2048 + lane * 16;
+  bf16x8 pcur[2], pnext[2];
+  dkdv_p_block(sQ, sLse, mine + pslot * kPBlockBytes, kf, lo, scale_log2, 0, hi, key_l, causal, pcur);
 #pragma unroll 1
   for (int nb = 0; nb < 4; ++nb) {     // 32 query rows at a time
-    const int blk = nb * 32 * kRowBytes;
-    int nat[8], trb[4][2];
-#pragma unroll
-    for (int ks = 0; ks < 8; ++ks) nat[ks] = lo.nat[ks] + blk;
-#pragma unroll
-    for (int mbd = 0; mbd < 4; ++mbd) { trb[mbd][0] = lo.tr[mbd][0] + blk; trb[mbd][1] = lo.tr[mbd][1] + blk; }
-    f32x16 s = f32x16{0};
-#pragma unroll
-    for (int ks = 0; ks < 8; ++ks) s = mfma32(lds_read_b128(sQ, nat[ks]), kf[ks], s);
-    // element i: query row 32*nb + 8*(i/4) + 4*hi + i%4, key column key_l
-    if (causal) {
-#pragma unroll
-      for (int i = 0; i < 16; ++i)
-        if (key_l > 32 * nb + 8 * (i >> 2) + 4 * hi + (i & 3)) s[i] = -INFINITY;
-    }
-    bf16x8 pb[2];
-#pragma unroll
-    for (int g = 0; g < 4; ++g) {
-      const f32x4 l4 = *reinterpret_cast<const f32x4*>(sLse + 32 * nb + 8 * g + 4 * hi);
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        const int i = 4 * g + j;
-        pb[i >> 3][i & 7] = (bf16)fast_exp2(fmaf(s[i], scale_log2, -l4[j]));
-      }
-    }
-    unsigned char* dst = sP + pbuf * kPBlockBytes + wave * 2048 + lane * 16;
-    *reinterpret_cast<bf16x8*>(dst) = pb[0];
-    *reinterpret_cast<bf16x8*>(dst + 1024) = pb[1];
-    pbuf ^= 1;
-    __syncthreads();                   // P of this block is visible to the partner wave
-#pragma unroll
-    for (int t = 0; t < 2; ++t)
-#pragma unroll
-      for (int mbd = 0; mbd < 4; ++mbd) {
-        const bf16x8 a_do = read_tr_pair(sdO + 16 * t * kRowBytes, trb[mbd][0], trb[mbd][1]);
-        dv[mbd] = mfma32(a_do, pb[t], dv[mbd]);
-      }
+    const int next_slot = pslot == 2 ? 0 : pslot + 1;
+    if (nb < 3) dkdv_p_block(sQ, sLse, mine + next_slot * kPBlockBytes, kf, lo, scale_log2, nb + 1, hi, key_l, causal, pnext);
+    pslot = next_slot;
+    lds_barrier();                     // P of block nb (and nb+1) is visible to the partner wave
+    mfma_tr_block(sdO, lo, nb * 32 * kRowBytes, pcur, dv);
+    pcur[0] = pnext[0];
+    pcur[1] = pnext[1];
   }
 }
 
 __device__ __forceinline__ void dkdv_tile_b(const unsigned char* sQ, const unsigned char* sdO, const float* sDelta,
-                                            const unsigned char* sP, int& pbuf, const bf16x8 (&vf)[8], f32x16 (&dk)[4],
+                                            const unsigned char* sP, int& pslot, const bf16x8 (&vf)[8], f32x16 (&dk)[4],
                                             const LaneOffsU& lo, int lane, int hi, int wave) {
 #pragma unroll 1
   for (int nb = 0; nb < 4; ++nb) {
     const int blk = nb * 32 * kRowBytes;
-    int nat[8], trb[4][2];
-#pragma unroll
-    for (int ks = 0; ks < 8; ++ks) nat[ks] = lo.nat[ks] + blk;
-#pragma unroll
-    for (int mbd = 0; mbd < 4; ++mbd) { trb[mbd][0] = lo.tr[mbd][0] + blk; trb[mbd][1] = lo.tr[mbd][1] + blk; }
-    f32x16 dp = f32x16{0};
-#pragma unroll
-    for (int ks = 0; ks < 8; ++ks) dp = mfma32(lds_read_b128(sdO, nat[ks]), vf[ks], dp);
-    __syncthreads();                   // the partner's P of this block has been written
-    const unsigned char* src = sP + pbuf * kPBlockBytes + wave * 2048 + lane * 16;
-    pbuf ^= 1;
+    const f32x16 dp = mfma_nat_block(sdO, lo, blk, vf);
+    lds_barrier();                     // the partner's P of this block has been written
+    const unsigned char* src = sP + pslot * kPBlockBytes + wave * 2048 + lane * 16;
+    pslot = pslot == 2 ? 0 : pslot + 1;
     u32x4 praw[2];
     praw[0] = *reinterpret_cast<const u32x4*>(src);
     praw[1] = *reinterpret_cast<const u32x4*>(src + 1024);
@@ -164,41 +194,23 @@ __device__ __forceinline__ void dkdv_tile_b(const unsigned char* sQ, const unsig
         dsb[i >> 3][i & 7] = (bf16)(pv * (dp[i] - d4[j]));
       }
     }
-#pragma unroll
-    for (int t = 0; t < 2; ++t)
-#pragma unroll
-      for (int mbd = 0; mbd < 4; ++mbd) {
-        const bf16x8 a_q = read_tr_pair(sQ + 16 * t * kRowBytes, trb[mbd][0], trb[mbd][1]);
-        dk[mbd] = mfma32(a_q, dsb[t], dk[mbd]);
-      }
+    mfma_tr_block(sQ, lo, blk, dsb, dk);
   }
 }
 
-__global__ __launch_bounds__(512) void dkdv_kernel(const BwdParams p) {
-  // two stages (Q tile, dO tile, the rows' lse and delta), distinct arrays per stage
-  __shared__ __attribute__((aligned(1024))) unsigned char sQ0[kTileBytes];
-  __shared__ __attribute__((aligned(1024))) unsigned char sdO0[kTileBytes];
-  __shared__ __attribute__((aligned(1024))) unsigned char sQ1[kTileBytes];
-  __shared__ __attribute__((aligned(1024))) unsigned char sdO1[kTileBytes];
-  __shared__ __attribute__((aligned(1024))) unsigned char sP[2 * kPBlockBytes];
-  __shared__ __attribute__((aligned(16))) float sStat0[2 * kTile];
-  __shared__ __attribute__((aligned(16))) float sStat1[2 * kTile];
+struct DkdvStage { unsigned char* q; unsigned char* dout; float* stat; };
 
-  const int tid = threadIdx.x, lane = tid & 63;
-  const int wave8 = __builtin_amdgcn_readfirstlane(tid >> 6);      // 0..7
-  const bool group_b = wave8 >= 4;
-  const int wave = wave8 & 3;
-  const int l32 = lane & 31, hi = lane >> 5;
-  int pos, bh;
-  map_block(blockIdx.x, p.batch * p.n_heads, p.heads_per_xcd, pos, bh);
-  const int kt = sload(p.order, pos);
-  const int b = bh / p.n_heads, h = bh % p.n_heads;
+// The whole key-tile column for one wave group (kGroupB: dK, else dV).  Both groups execute the
+// same sequence of barriers.
+template <bool kGroupB>
+__device__ __forceinline__ void dkdv_run(const BwdParams& p, const DkdvStage (&stg)[2], unsigned char* sP, int kt, int b,
+                                         int h, int tid, int lane, int wave8) {
+  const int wave = wave8 & 3, l32 = lane & 31, hi = lane >> 5;
   const int64_t seq_q = (int64_t)p.n_qtiles * kTile;
-
   // group A keeps the K fragments, group B the V fragments (B operands): lane holds key row
   // 32*wave + lane%32, d = 16*ks + 8*hi .. +7
   const int krow = kt * kTile + wave * 32 + l32;
-  const bf16* fp = group_b ? p.v + b * p.vs.b + (int64_t)krow * p.vs.s + h * p.vs.h + hi * 8
+  const bf16* fp = kGroupB ? p.v + b * p.vs.b + (int64_t)krow * p.vs.s + h * p.vs.h + hi * 8
                            : p.k + b * p.ks.b + (int64_t)krow * p.ks.s + h * p.ks.h + hi * 8;
   bf16x8 frag[8];
 #pragma unroll
@@ -233,28 +245,32 @@ __global__ __launch_bounds__(512) void dkdv_kernel(const BwdParams p) {
     }
     return x;
   };
-  auto stage = [&](int qt, unsigned char* sQ, unsigned char* sdO) {
+  auto stage = [&](int qt, const DkdvStage& st) {
     const __amdgpu_buffer_rsrc_t rq = make_rsrc(qbase + (int64_t)qt * kTile * q_stride, q_extent);
     const __amdgpu_buffer_rsrc_t rd = make_rsrc(dobase + (int64_t)qt * kTile * do_stride, do_extent);
-    dma_half_tile_buf<8>(sQ, rq, qoff, 0, wave8);
-    dma_half_tile_buf<8>(sQ + kHalfBytes, rq, qoff, q_half, wave8);
-    dma_half_tile_buf<8>(sdO, rd, dooff, 0, wave8);
-    dma_half_tile_buf<8>(sdO + kHalfBytes, rd, dooff, do_half, wave8);
+    dma_half_tile_buf<8>(st.q, rq, qoff, 0, wave8);
+    dma_half_tile_buf<8>(st.q + kHalfBytes, rq, qoff, q_half, wave8);
+    dma_half_tile_buf<8>(st.dout, rd, dooff, 0, wave8);
+    dma_half_tile_buf<8>(st.dout + kHalfBytes, rd, dooff, do_half, wave8);
   };
-  auto tile = [&](const unsigned char* sQ, const unsigned char* sdO, const float* sStat, int& pbuf, bool causal) {
-    if (group_b) dkdv_tile_b(sQ, sdO, sStat + kTile, sP, pbuf, frag, acc, lo, lane, hi, wave);
-    else         dkdv_tile_a(sQ, sdO, sStat, sP, pbuf, frag, acc, lo, p.scale_log2, lane, hi, wave, key_l, causal);
+  // Both groups advance the hand-over slot once per block: group A names the slot of the block
+  // it writes next (one ahead), group B the slot of the block it reads.
+  int pslot = 0;
+  auto tile = [&](const DkdvStage& st, bool causal) {
+    if (kGroupB) dkdv_tile_b(st.q, st.dout, st.stat + kTile, sP, pslot, frag, acc, lo, lane, hi, wave);
+    else         dkdv_tile_a(st.q, st.dout, st.stat, sP, pslot, frag, acc, lo, p.scale_log2, lane, hi, wave, key_l, causal);
   };
 
   const int e0 = sload(p.ptr, kt), e1 = sload(p.ptr, kt + 1);
   if (e0 < e1) {
     const int qt = qtile(e0);
     const float st0 = load_stat(qt);
-    if (tid < 2 * kTile) sStat0[tid] = st0;
-    stage(qt, sQ0, sdO0);
+    if (tid < 2 * kTile) stg[0].stat[tid] = st0;
+    stage(qt, stg[0]);
   }
-  int pbuf = 0;
-  // entries are taken two at a time: even ones through stage 0, odd ones through stage 1
+  // entries are taken two at a time, even ones through stage 0 and odd ones through stage 1,
+  // so that every LDS access names its stage statically (reads of one stage then need not
+  // wait for the copies in flight into the other)
   for (int e = e0; e < e1; e += 2) {
     const bool has1 = e + 1 < e1, has2 = e + 2 < e1;
     float stat = 0.f;
@@ -263,23 +279,44 @@ __global__ __launch_bounds__(512) void dkdv_kernel(const BwdParams p) {
     if (has1) {
       const int qt = qtile(e + 1);
       stat = load_stat(qt);
-      stage(qt, sQ1, sdO1);
+      stage(qt, stg[1]);
     }
-    tile(sQ0, sdO0, sStat0, pbuf, sload(p.flag, e) != 0);
+    tile(stg[0], sload(p.flag, e) != 0);
     if (!has1) break;
-    if (tid < 2 * kTile) sStat1[tid] = stat;
+    if (tid < 2 * kTile) stg[1].stat[tid] = stat;
     wait_vmem_all();
     __syncthreads();                       // stage 1 landed; everyone is done with stage 0
     if (has2) {
       const int qt = qtile(e + 2);
       stat = load_stat(qt);
-      stage(qt, sQ0, sdO0);
+      stage(qt, stg[0]);
     }
-    tile(sQ1, sdO1, sStat1, pbuf, sload(p.flag, e + 1) != 0);
-    if (has2 && tid < 2 * kTile) sStat0[tid] = stat;
+    tile(stg[1], sload(p.flag, e + 1) != 0);
+    if (has2 && tid < 2 * kTile) stg[0].stat[tid] = stat;
   }
-  if (group_b) store_acc_t(p.out0 + b * p.o0s.b + (int64_t)krow * p.o0s.s + h * p.o0s.h, acc, p.scale, hi);
+  if (kGroupB) store_acc_t(p.out0 + b * p.o0s.b + (int64_t)krow * p.o0s.s + h * p.o0s.h, acc, p.scale, hi);
   else         store_acc_t(p.out1 + b * p.o1s.b + (int64_t)krow * p.o1s.s + h * p.o1s.h, acc, 1.f, hi);
+}
+
+__global__ __launch_bounds__(512) void dkdv_kernel(const BwdParams p) {
+  // two stages (Q tile, dO tile, the rows' lse and delta)
+  __shared__ __attribute__((aligned(1024))) unsigned char sQ0[kTileBytes];
+  __shared__ __attribute__((aligned(1024))) unsigned char sdO0[kTileBytes];
+  __shared__ __attribute__((aligned(1024))) unsigned char sQ1[kTileBytes];
+  __shared__ __attribute__((aligned(1024))) unsigned char sdO1[kTileBytes];
+  __shared__ __attribute__((aligned(1024))) unsigned char sP[3 * kPBlockBytes];
+  __shared__ __attribute__((aligned(16))) float sStat0[2 * kTile];
+  __shared__ __attribute__((aligned(16))) float sStat1[2 * kTile];
+
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave8 = __builtin_amdgcn_readfirstlane(tid >> 6);      // 0..7
+  int pos, bh;
+  map_block(blockIdx.x, p.batch * p.n_heads, p.heads_per_xcd, pos, bh);
+  const int kt = sload(p.order, pos);
+  const int b = bh / p.n_heads, h = bh % p.n_heads;
+  const DkdvStage stg[2] = {{sQ0, sdO0, sStat0}, {sQ1, sdO1, sStat1}};
+  if (wave8 >= 4) dkdv_run<true>(p, stg, sP, kt, b, h, tid, lane, wave8);
+  else            dkdv_run<false>(p, stg, sP, kt, b, h, tid, lane, wave8);
 }
 
 // dQ: one 64-key half tile for this wave's 32 query rows.

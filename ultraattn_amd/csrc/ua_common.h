@@ -108,6 +108,11 @@ __device__ __forceinline__ void dma16(const bf16* gsrc, unsigned char* lds_dst) 
                                    (__attribute__((address_space(3))) void*)lds_dst, 16, 0, 0);
 }
 __device__ __forceinline__ void wait_vmem_all() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
+// Workgroup barrier that orders LDS traffic only: unlike __syncthreads() it does not wait for
+// the asynchronous global->LDS copies still in flight (they target another stage).
+__device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
+// Keeps a wave-uniform branch a branch (the optimiser may not turn its body into selects).
+__device__ __forceinline__ void keep_branch() { asm volatile("" ::: "memory"); }
 
 // Per-thread source offsets (in elements) for staging a [64][128] bf16 half tile (16 KiB) with
 // NW waves: each thread issues 16/NW DMA instructions; instruction i of wave w fills LDS rows
