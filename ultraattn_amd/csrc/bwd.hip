@@ -108,25 +108,29 @@ __device__ __forceinline__ void mfma_tr_block(const unsigned char* sX, const Lan
   }
 }
 
-// One 32x32 block X[rows 32*nb.., :] * frag^T over head_dim: the 8 row fragments are all fetched
-// before the dependent MFMA chain starts.
+// One 32x32 block X[rows 32*nb.., :] * frag^T over head_dim: the row fragments are fetched
+// kAhead reads ahead of the (dependent) MFMA chain.
 __device__ __forceinline__ f32x16 mfma_nat_block(const unsigned char* sX, const LaneOffsU& lo, int blk,
                                                  const bf16x8 (&frag)[8]) {
+  constexpr int kAhead = 4;
   bf16x8 fr[8];
 #pragma unroll
-  for (int ks = 0; ks < 8; ++ks) fr[ks] = lds_read_b128(sX, lo.nat[ks] + blk);
-  __builtin_amdgcn_sched_group_barrier(0x100, 8, 0);
+  for (int ks = 0; ks < kAhead; ++ks) fr[ks] = lds_read_b128(sX, lo.nat[ks] + blk);
+  __builtin_amdgcn_sched_group_barrier(0x100, kAhead, 0);
   f32x16 acc = f32x16{0};
 #pragma unroll
-  for (int ks = 0; ks < 8; ++ks) acc = mfma32(fr[ks], frag[ks], acc);
+  for (int ks = 0; ks < 8; ++ks) {
+    if (ks + kAhead < 8) fr[ks + kAhead] = lds_read_b128(sX, lo.nat[ks + kAhead] + blk);
+    acc = mfma32(fr[ks], frag[ks], acc);
+    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+    __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+  }
   return acc;
 }
 
-// S^T block -> P (bf16, accumulator layout) for query rows 32*nb.., written to the hand-over slot.
-__device__ __forceinline__ void dkdv_p_block(const unsigned char* sQ, const float* sLse, unsigned char* p_slot,
-                                             const bf16x8 (&kf)[8], const LaneOffsU& lo, float scale_log2, int nb,
-                                             int hi, int key_l, bool causal, bf16x8 (&pb)[2]) {
-  f32x16 s = mfma_nat_block(sQ, lo, nb * 32 * kRowBytes, kf);
+// P = exp2(scale*S - lse) for one block (bf16, accumulator layout), written to the hand-over slot.
+__device__ __forceinline__ void dkdv_p_from_s(f32x16 s, const f32x4 (&lse4)[4], unsigned char* p_slot, float scale_log2,
+                                              int nb, int hi, int key_l, bool causal, bf16x8 (&pb)[2]) {
   // element i: query row 32*nb + 8*(i/4) + 4*hi + i%4, key column key_l
   if (causal) {
     keep_branch();
@@ -135,66 +139,66 @@ __device__ __forceinline__ void dkdv_p_block(const unsigned char* sQ, const floa
       if (key_l > 32 * nb + 8 * (i >> 2) + 4 * hi + (i & 3)) s[i] = -INFINITY;
   }
 #pragma unroll
-  for (int g = 0; g < 4; ++g) {
-    const f32x4 l4 = *reinterpret_cast<const f32x4*>(sLse + 32 * nb + 8 * g + 4 * hi);
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      const int i = 4 * g + j;
-      pb[i >> 3][i & 7] = (bf16)fast_exp2(fmaf(s[i], scale_log2, -l4[j]));
-    }
-  }
+  for (int i = 0; i < 16; ++i)
+    pb[i >> 3][i & 7] = (bf16)fast_exp2(fmaf(s[i], scale_log2, -lse4[i >> 2][i & 3]));
   *reinterpret_cast<bf16x8*>(p_slot) = pb[0];
   *reinterpret_cast<bf16x8*>(p_slot + 1024) = pb[1];
 }
 
-// Group A runs one block ahead of its partner: P of block nb+1 is produced before the
-// workgroup barrier of block nb, so its exp2 work overlaps the partner's MFMAs.  Three hand-over
-// slots: P(nb+2) may be written while the partner still reads P(nb).
+__device__ __forceinline__ void load_stat4(const float* sStat, int nb, int hi, f32x4 (&v)[4]) {
+#pragma unroll
+  for (int g = 0; g < 4; ++g) v[g] = *reinterpret_cast<const f32x4*>(sStat + 32 * nb + 8 * g + 4 * hi);
+}
+
+// Group A, one query tile.  Software pipelined inside the wave: the MFMAs of S(nb+1) are issued
+// first and run while the vector unit turns S(nb) into P(nb); then the barrier publishes P(nb)
+// and dV takes it.
 __device__ __forceinline__ void dkdv_tile_a(const unsigned char* sQ, const unsigned char* sdO, const float* sLse,
                                             unsigned char* sP, int& pslot, const bf16x8 (&kf)[8], f32x16 (&dv)[4],
                                             const LaneOffsU& lo, float scale_log2, int lane, int hi, int wave,
                                             int key_l, bool causal) {
   unsigned char* mine = sP + wave * 2048 + lane * 16;
-  bf16x8 pcur[2], pnext[2];
-  dkdv_p_block(sQ, sLse, mine + pslot * kPBlockBytes, kf, lo, scale_log2, 0, hi, key_l, causal, pcur);
-#pragma unroll 1
+  f32x16 s_cur = mfma_nat_block(sQ, lo, 0, kf), s_next;
+  bf16x8 pb[2];
+  f32x4 lse4[4];
+#pragma unroll
   for (int nb = 0; nb < 4; ++nb) {     // 32 query rows at a time
-    const int next_slot = pslot == 2 ? 0 : pslot + 1;
-    if (nb < 3) dkdv_p_block(sQ, sLse, mine + next_slot * kPBlockBytes, kf, lo, scale_log2, nb + 1, hi, key_l, causal, pnext);
-    pslot = next_slot;
-    lds_barrier();                     // P of block nb (and nb+1) is visible to the partner wave
-    mfma_tr_block(sdO, lo, nb * 32 * kRowBytes, pcur, dv);
-    pcur[0] = pnext[0];
-    pcur[1] = pnext[1];
+    load_stat4(sLse, nb, hi, lse4);
+    if (nb < 3) s_next = mfma_nat_block(sQ, lo, (nb + 1) * 32 * kRowBytes, kf);
+    dkdv_p_from_s(s_cur, lse4, mine + pslot * kPBlockBytes, scale_log2, nb, hi, key_l, causal, pb);
+    pslot = pslot == 2 ? 0 : pslot + 1;
+    lds_barrier();                     // P of block nb is visible to the partner wave
+    mfma_tr_block(sdO, lo, nb * 32 * kRowBytes, pb, dv);
+    s_cur = s_next;
   }
 }
 
+// Group B, one query tile: dP(nb+1)'s MFMAs run while dS(nb) = P(nb) * (dP(nb) - delta) is formed.
 __device__ __forceinline__ void dkdv_tile_b(const unsigned char* sQ, const unsigned char* sdO, const float* sDelta,
                                             const unsigned char* sP, int& pslot, const bf16x8 (&vf)[8], f32x16 (&dk)[4],
                                             const LaneOffsU& lo, int lane, int hi, int wave) {
-#pragma unroll 1
+  const unsigned char* mine = sP + wave * 2048 + lane * 16;
+  f32x16 dp_cur = mfma_nat_block(sdO, lo, 0, vf), dp_next;
+  f32x4 d4[4];
+#pragma unroll
   for (int nb = 0; nb < 4; ++nb) {
-    const int blk = nb * 32 * kRowBytes;
-    const f32x16 dp = mfma_nat_block(sdO, lo, blk, vf);
+    load_stat4(sDelta, nb, hi, d4);
+    if (nb < 3) dp_next = mfma_nat_block(sdO, lo, (nb + 1) * 32 * kRowBytes, vf);
     lds_barrier();                     // the partner's P of this block has been written
-    const unsigned char* src = sP + pslot * kPBlockBytes + wave * 2048 + lane * 16;
+    const unsigned char* src = mine + pslot * kPBlockBytes;
     pslot = pslot == 2 ? 0 : pslot + 1;
     u32x4 praw[2];
     praw[0] = *reinterpret_cast<const u32x4*>(src);
     praw[1] = *reinterpret_cast<const u32x4*>(src + 1024);
     bf16x8 dsb[2];
 #pragma unroll
-    for (int g = 0; g < 4; ++g) {
-      const f32x4 d4 = *reinterpret_cast<const f32x4*>(sDelta + 32 * nb + 8 * g + 4 * hi);
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        const int i = 4 * g + j;
-        const uint32_t w = praw[i >> 3][(i & 7) >> 1];
-        const float pv = __uint_as_float((i & 1) ? (w & 0xffff0000u) : (w << 16));
-        dsb[i >> 3][i & 7] = (bf16)(pv * (dp[i] - d4[j]));
-      }
+    for (int i = 0; i < 16; ++i) {
+      const uint32_t w = praw[i >> 3][(i & 7) >> 1];
+      const float pv = __uint_as_float((i & 1) ? (w & 0xffff0000u) : (w << 16));
+      dsb[i >> 3][i & 7] = (bf16)(pv * (dp_cur[i] - d4[i >> 2][i & 3]));
     }
-    mfma_tr_block(sQ, lo, blk, dsb, dk);
+    mfma_tr_block(sQ, lo, nb * 32 * kRowBytes, dsb, dk);
+    dp_cur = dp_next;
   }
 }
 
