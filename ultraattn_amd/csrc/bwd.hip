@@ -330,16 +330,35 @@ __device__ __forceinline__ void dq_half_tile(const unsigned char* sK, const unsi
                                              int key0, bool mask) {
 #pragma unroll
   for (int mb = 0; mb < 2; ++mb) {     // 32 keys at a time
+    // S^T and dP^T blocks: 16 row fragments (K and V alternating), fetched kAhead reads ahead
     f32x16 s = f32x16{0}, dp = f32x16{0};
+    {
+      constexpr int kAhead = 4;
+      bf16x8 fr[16];
+      auto rd = [&](int i) {
+        return (i & 1) ? lds_read_b128(sV, lds_off_k(32 * mb + l32, 2 * (i >> 1) + hi))
+                       : lds_read_b128(sK, lds_off_u(32 * mb + l32, 2 * (i >> 1) + hi));
+      };
 #pragma unroll
-    for (int ks = 0; ks < 8; ++ks) {
-      const bf16x8 ak = lds_read_b128(sK, lds_off_u(32 * mb + l32, 2 * ks + hi));
-      s = mfma32(ak, qf[ks], s);
-      const bf16x8 av = lds_read_b128(sV, lds_off_k(32 * mb + l32, 2 * ks + hi));
-      dp = mfma32(av, dof[ks], dp);
+      for (int i = 0; i < kAhead; ++i) fr[i] = rd(i);
+      __builtin_amdgcn_sched_group_barrier(0x100, kAhead, 0);
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        if (i + kAhead < 16) fr[i + kAhead] = rd(i + kAhead);
+        if (i & 1) dp = mfma32(fr[i], dof[i >> 1], dp);
+        else       s = mfma32(fr[i], qf[i >> 1], s);
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+      }
     }
+    // the first K^T fragments of the dQ product are fetched now, behind the pointwise work
+    constexpr int kTAhead = 3;
+    bf16x8 tfr[8];
+#pragma unroll
+    for (int i = 0; i < kTAhead; ++i) tfr[i] = lds_read_tr_frag<lds_off_u>(sK, tr, 32 * mb + 16 * (i >> 2), i & 3);
     // element i: key key0 + 32*mb + 8*(i/4) + 4*hi + i%4, query column q_l
     if (mask) {
+      keep_branch();
 #pragma unroll
       for (int i = 0; i < 16; ++i)
         if (key0 + 32 * mb + 8 * (i >> 2) + 4 * hi + (i & 3) > q_l) s[i] = -INFINITY;
@@ -351,12 +370,12 @@ __device__ __forceinline__ void dq_half_tile(const unsigned char* sK, const unsi
       dsb[i >> 3][i & 7] = (bf16)(pv * (dp[i] - delta));
     }
 #pragma unroll
-    for (int t = 0; t < 2; ++t)
-#pragma unroll
-      for (int mbd = 0; mbd < 4; ++mbd) {
-        const bf16x8 a_k = lds_read_tr_frag<lds_off_u>(sK, tr, 32 * mb + 16 * t, mbd);
-        dq[mbd] = mfma32(a_k, dsb[t], dq[mbd]);
-      }
+    for (int i = 0; i < 8; ++i) {
+      if (i + kTAhead < 8) tfr[i + kTAhead] = lds_read_tr_frag<lds_off_u>(sK, tr, 32 * mb + 16 * ((i + kTAhead) >> 2), (i + kTAhead) & 3);
+      dq[i & 3] = mfma32(tfr[i], dsb[i >> 2], dq[i & 3]);
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+    }
   }
 }
 
