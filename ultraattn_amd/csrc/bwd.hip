@@ -108,16 +108,24 @@ __device__ __forceinline__ void mfma_tr_block(const unsigned char* sX, const Lan
   }
 }
 
-// One 32x32 block X[rows 32*nb.., :] * frag^T over head_dim: the row fragments are fetched
-// kAhead reads ahead of the (dependent) MFMA chain.
+// One 32x32 block: stat + X[rows 32*nb.., :] * frag^T over head_dim.  The accumulator starts
+// from the rows' statistic (4 x 128-bit LDS reads straight into it) instead of zero, which
+// folds the "- lse" / "- delta" of the pointwise step into the product.  The row fragments
+// are fetched kAhead reads ahead of the (dependent) MFMA chain.
 __device__ __forceinline__ f32x16 mfma_nat_block(const unsigned char* sX, const LaneOffsU& lo, int blk,
-                                                 const bf16x8 (&frag)[8]) {
+                                                 const bf16x8 (&frag)[8], const float* stat_rows, int hi) {
   constexpr int kAhead = 4;
   bf16x8 fr[8];
 #pragma unroll
   for (int ks = 0; ks < kAhead; ++ks) fr[ks] = lds_read_b128(sX, lo.nat[ks] + blk);
-  __builtin_amdgcn_sched_group_barrier(0x100, kAhead, 0);
-  f32x16 acc = f32x16{0};
+  f32x16 acc;
+  // element i: row 8*(i/4) + 4*hi + i%4 of the block
+#pragma unroll
+  for (int g = 0; g < 4; ++g) {
+    const f32x4 v = *reinterpret_cast<const f32x4*>(stat_rows + 8 * g + 4 * hi);
+    acc[4 * g] = v[0]; acc[4 * g + 1] = v[1]; acc[4 * g + 2] = v[2]; acc[4 * g + 3] = v[3];
+  }
+  __builtin_amdgcn_sched_group_barrier(0x100, kAhead + 4, 0);
 #pragma unroll
   for (int ks = 0; ks < 8; ++ks) {
     if (ks + kAhead < 8) fr[ks + kAhead] = lds_read_b128(sX, lo.nat[ks + kAhead] + blk);
@@ -128,8 +136,9 @@ __device__ __forceinline__ f32x16 mfma_nat_block(const unsigned char* sX, const 
   return acc;
 }
 
-// P = exp2(scale*S - lse) for one block (bf16, accumulator layout), written to the hand-over slot.
-__device__ __forceinline__ void dkdv_p_from_s(f32x16 s, const f32x4 (&lse4)[4], unsigned char* p_slot, float scale_log2,
+// P = exp2(scale_log2 * S') with S' = Q K^T - lse/scale (bf16, accumulator layout), written to
+// the hand-over slot.
+__device__ __forceinline__ void dkdv_p_from_s(f32x16 s, unsigned char* p_slot, float scale_log2,
                                               int nb, int hi, int key_l, bool causal, bf16x8 (&pb)[2]) {
   // element i: query row 32*nb + 8*(i/4) + 4*hi + i%4, key column key_l
   if (causal) {
@@ -139,33 +148,24 @@ __device__ __forceinline__ void dkdv_p_from_s(f32x16 s, const f32x4 (&lse4)[4], 
       if (key_l > 32 * nb + 8 * (i >> 2) + 4 * hi + (i & 3)) s[i] = -INFINITY;
   }
 #pragma unroll
-  for (int i = 0; i < 16; ++i)
-    pb[i >> 3][i & 7] = (bf16)fast_exp2(fmaf(s[i], scale_log2, -lse4[i >> 2][i & 3]));
+  for (int i = 0; i < 16; ++i) pb[i >> 3][i & 7] = (bf16)fast_exp2(s[i] * scale_log2);
   *reinterpret_cast<bf16x8*>(p_slot) = pb[0];
   *reinterpret_cast<bf16x8*>(p_slot + 1024) = pb[1];
 }
 
-__device__ __forceinline__ void load_stat4(const float* sStat, int nb, int hi, f32x4 (&v)[4]) {
-#pragma unroll
-  for (int g = 0; g < 4; ++g) v[g] = *reinterpret_cast<const f32x4*>(sStat + 32 * nb + 8 * g + 4 * hi);
-}
-
-// Group A, one query tile.  Software pipelined inside the wave: the MFMAs of S(nb+1) are issued
-// first and run while the vector unit turns S(nb) into P(nb); then the barrier publishes P(nb)
-// and dV takes it.
+// Group A, one query tile.  The MFMAs of S(nb+1) are issued before the vector unit turns S(nb)
+// into P(nb); then the barrier publishes P(nb) and dV takes it.
 __device__ __forceinline__ void dkdv_tile_a(const unsigned char* sQ, const unsigned char* sdO, const float* sLse,
                                             unsigned char* sP, int& pslot, const bf16x8 (&kf)[8], f32x16 (&dv)[4],
                                             const LaneOffsU& lo, float scale_log2, int lane, int hi, int wave,
                                             int key_l, bool causal) {
   unsigned char* mine = sP + wave * 2048 + lane * 16;
-  f32x16 s_cur = mfma_nat_block(sQ, lo, 0, kf), s_next;
+  f32x16 s_cur = mfma_nat_block(sQ, lo, 0, kf, sLse, hi), s_next;
   bf16x8 pb[2];
-  f32x4 lse4[4];
 #pragma unroll
   for (int nb = 0; nb < 4; ++nb) {     // 32 query rows at a time
-    load_stat4(sLse, nb, hi, lse4);
-    if (nb < 3) s_next = mfma_nat_block(sQ, lo, (nb + 1) * 32 * kRowBytes, kf);
-    dkdv_p_from_s(s_cur, lse4, mine + pslot * kPBlockBytes, scale_log2, nb, hi, key_l, causal, pb);
+    if (nb < 3) s_next = mfma_nat_block(sQ, lo, (nb + 1) * 32 * kRowBytes, kf, sLse + 32 * (nb + 1), hi);
+    dkdv_p_from_s(s_cur, mine + pslot * kPBlockBytes, scale_log2, nb, hi, key_l, causal, pb);
     pslot = pslot == 2 ? 0 : pslot + 1;
     lds_barrier();                     // P of block nb is visible to the partner wave
     mfma_tr_block(sdO, lo, nb * 32 * kRowBytes, pb, dv);
@@ -173,17 +173,16 @@ __device__ __forceinline__ void dkdv_tile_a(const unsigned char* sQ, const unsig
   }
 }
 
-// Group B, one query tile: dP(nb+1)'s MFMAs run while dS(nb) = P(nb) * (dP(nb) - delta) is formed.
-__device__ __forceinline__ void dkdv_tile_b(const unsigned char* sQ, const unsigned char* sdO, const float* sDelta,
+// Group B, one query tile: dP'(nb+1) = dO V^T - delta is issued before dS(nb) = P(nb) * dP'(nb)
+// is formed.
+__device__ __forceinline__ void dkdv_tile_b(const unsigned char* sQ, const unsigned char* sdO, const float* sNegDelta,
                                             const unsigned char* sP, int& pslot, const bf16x8 (&vf)[8], f32x16 (&dk)[4],
                                             const LaneOffsU& lo, int lane, int hi, int wave) {
   const unsigned char* mine = sP + wave * 2048 + lane * 16;
-  f32x16 dp_cur = mfma_nat_block(sdO, lo, 0, vf), dp_next;
-  f32x4 d4[4];
+  f32x16 dp_cur = mfma_nat_block(sdO, lo, 0, vf, sNegDelta, hi), dp_next;
 #pragma unroll
   for (int nb = 0; nb < 4; ++nb) {
-    load_stat4(sDelta, nb, hi, d4);
-    if (nb < 3) dp_next = mfma_nat_block(sdO, lo, (nb + 1) * 32 * kRowBytes, vf);
+    if (nb < 3) dp_next = mfma_nat_block(sdO, lo, (nb + 1) * 32 * kRowBytes, vf, sNegDelta + 32 * (nb + 1), hi);
     lds_barrier();                     // the partner's P of this block has been written
     const unsigned char* src = mine + pslot * kPBlockBytes;
     pslot = pslot == 2 ? 0 : pslot + 1;
@@ -195,7 +194,7 @@ __device__ __forceinline__ void dkdv_tile_b(const unsigned char* sQ, const unsig
     for (int i = 0; i < 16; ++i) {
       const uint32_t w = praw[i >> 3][(i & 7) >> 1];
       const float pv = __uint_as_float((i & 1) ? (w & 0xffff0000u) : (w << 16));
-      dsb[i >> 3][i & 7] = (bf16)(pv * (dp_cur[i] - d4[i >> 2][i & 3]));
+      dsb[i >> 3][i & 7] = (bf16)(pv * dp_cur[i]);
     }
     mfma_tr_block(sQ, lo, nb * 32 * kRowBytes, dsb, dk);
     dp_cur = dp_next;
@@ -239,13 +238,15 @@ __device__ __forceinline__ void dkdv_run(const BwdParams& p, const DkdvStage (&s
   const uint32_t q_extent = (uint32_t)((kTile - 1) * q_stride + kHeadDim) * 2;
   const uint32_t do_extent = (uint32_t)((kTile - 1) * do_stride + kHeadDim) * 2;
   auto qtile = [&](int e) { return min(max(sload(p.idx, e), 0), p.n_qtiles - 1); };
-  // rows' statistics: threads 0..127 carry lse (pre-multiplied by log2 e; -inf -> +inf so that
-  // rows without keys give P = 0), threads 128..255 carry delta
+  // rows' statistics, staged in the form the accumulators start from: threads 0..127 carry
+  // -lse/softmax_scale (lse = -inf, a row without keys, stays -inf so that P = 0), threads
+  // 128..255 carry -delta
+  const float neg_inv_scale = -1.f / p.scale;
   auto load_stat = [&](int qt) {
     float x = 0.f;
     if (tid < 2 * kTile) {
       x = tid < kTile ? lse_row[qt * kTile + tid] : delta_row[qt * kTile + tid - kTile];
-      if (tid < kTile) x = (x == -INFINITY) ? INFINITY : x * kLog2e;
+      x = tid < kTile ? ((x == -INFINITY) ? -INFINITY : x * neg_inv_scale) : -x;
     }
     return x;
   };
