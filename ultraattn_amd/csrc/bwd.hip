@@ -327,12 +327,15 @@ __global__ __launch_bounds__(512) void dkdv_kernel(const BwdParams p) {
 // dQ: one 64-key half tile for this wave's 32 query rows.
 __device__ __forceinline__ void dq_half_tile(const unsigned char* sK, const unsigned char* sV, const bf16x8 (&qf)[8],
                                              const bf16x8 (&dof)[8], f32x16 (&dq)[4], const TrLane& tr,
-                                             float scale_log2, float lse2, float delta, int l32, int hi, int q_l,
+                                             float scale_log2, float lse2, float neg_delta, int l32, int hi, int q_l,
                                              int key0, bool mask) {
 #pragma unroll
   for (int mb = 0; mb < 2; ++mb) {     // 32 keys at a time
     // S^T and dP^T blocks: 16 row fragments (K and V alternating), fetched kAhead reads ahead
-    f32x16 s = f32x16{0}, dp = f32x16{0};
+    // dP' = V dO^T - delta: the accumulator starts from -delta (a per-lane scalar here)
+    f32x16 s = f32x16{0}, dp;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) dp[i] = neg_delta;
     {
       constexpr int kAhead = 4;
       bf16x8 fr[16];
@@ -368,7 +371,7 @@ __device__ __forceinline__ void dq_half_tile(const unsigned char* sK, const unsi
 #pragma unroll
     for (int i = 0; i < 16; ++i) {
       const float pv = fast_exp2(fmaf(s[i], scale_log2, -lse2));
-      dsb[i >> 3][i & 7] = (bf16)(pv * (dp[i] - delta));
+      dsb[i >> 3][i & 7] = (bf16)(pv * dp[i]);
     }
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
@@ -427,7 +430,7 @@ __global__ __launch_bounds__(256, 2) void dq_kernel(const BwdParams p) {
   }
   const float lse_raw = p.lse[((int64_t)b * p.n_heads + h) * seq_q + qrow];
   const float lse2 = (lse_raw == -INFINITY) ? INFINITY : lse_raw * kLog2e;
-  const float delta = p.delta[((int64_t)b * p.n_heads + h) * seq_q + qrow];
+  const float neg_delta = -p.delta[((int64_t)b * p.n_heads + h) * seq_q + qrow];
 
   f32x16 dq[4];
 #pragma unroll
@@ -442,7 +445,7 @@ __global__ __launch_bounds__(256, 2) void dq_kernel(const BwdParams p) {
     dma_half_tile_buf<4>(sKB, k_rsrc(kt), koff, k_half, wave);
     dma_half_tile_buf<4>(sVB, v_rsrc(kt), voff, v_half, wave);
     // causal tile: queries 64..127 (waves 2, 3) see all of keys 0..63
-    dq_half_tile(sKA, sVA, qf, dof, dq, tr, p.scale_log2, lse2, delta, l32, hi, q_l, 0, causal && wave < 2);
+    dq_half_tile(sKA, sVA, qf, dof, dq, tr, p.scale_log2, lse2, neg_delta, l32, hi, q_l, 0, causal && wave < 2);
     wait_vmem_all();
     __syncthreads();            // stage B landed; everyone is done with stage A
     if (e + 1 < e1) {
@@ -451,7 +454,7 @@ __global__ __launch_bounds__(256, 2) void dq_kernel(const BwdParams p) {
     }
     // causal tile: queries 0..63 (waves 0, 1) see none of keys 64..127
     if (!causal || wave >= 2)
-      dq_half_tile(sKB, sVB, qf, dof, dq, tr, p.scale_log2, lse2, delta, l32, hi, q_l, kHalf, causal);
+      dq_half_tile(sKB, sVB, qf, dof, dq, tr, p.scale_log2, lse2, neg_delta, l32, hi, q_l, kHalf, causal);
     kt = kt_next;
   }
   store_acc_t(p.out0 + b * p.o0s.b + (int64_t)qrow * p.o0s.s + h * p.o0s.h, dq, p.scale, hi);
