@@ -10,4 +10,7 @@ def __getattr__(name):
     if name in ("bsa_fwd", "bsa_bwd", "merge_partials", "softmax_delta"):
         from . import ops
         return getattr(ops, name)
+    if name in ("BlockSparseExecutor", "mask_from_comp_kernels", "comp_kernels_from_schedule"):
+        from . import executor
+        return getattr(executor, name)
     raise AttributeError(name)

@@ -1,0 +1,133 @@
+"""One-GPU counterpart of the reference's plan-driven loop over ``Comp_Kernel``s
+(``intra_attn_forward`` / ``intra_attn_backward``,
+``orchestrated_attn/orchestrated_attn_impl.py:300-363, 554-620``).
+
+The reference walks ``execution_plan.gpu_kernel_lists[rank]`` and launches one dense
+flash-attention call per ``Comp_Kernel`` key ``(b, h, r_id | r_ids, c_id | c_ids, gpu)``
+(``search_algo/dependent_graph.py:51-72``; fused rectangles carry tuples of ids,
+``search_algo/graph_transformation_engine.py:83``).  Here the same list becomes ONE block mask,
+hence one tile list and one kernel launch per direction, and the ``reduce`` steps the reference
+leaves as stubs (``orchestrated_attn/utils.py:119-134, 260-262, 296-298``) are the merge kernel
+and an fp32 sum.
+"""
+from typing import Iterable, List, Optional, Sequence, Tuple, Union
+
+import numpy as np
+import torch
+
+from .masks import CAUSAL, EMPTY, FULL
+from .ops import bsa_bwd, bsa_fwd, merge_partials, softmax_delta
+from .tilelist import TileList, build_tile_list
+
+Ids = Union[int, Tuple[int, ...]]
+CompKey = Tuple[int, int, Ids, Ids, int]
+
+
+def _ids(x: Ids) -> Tuple[int, ...]:
+    return tuple(int(i) for i in x) if isinstance(x, (tuple, list, np.ndarray)) else (int(x),)
+
+
+def mask_from_comp_kernels(keys: Iterable[CompKey], n_row_chunks: int, n_col_chunks: int, causal: bool,
+                           rank: Optional[int] = None) -> np.ndarray:
+    """Block mask (0/1/2) covered by a list of ``Comp_Kernel`` keys.  A kernel is causal iff the
+    mask is causal and its row id is a plain int equal to its column id
+    (``kernel_causal = causal and isinstance(rid, int) and rid == cid``,
+    ``orchestrated_attn_impl.py:91``); a fused rectangle (tuple ids) is a dense block of chunks.
+    ``rank`` keeps only the keys assigned to that GPU (key[4])."""
+    m = np.zeros((n_row_chunks, n_col_chunks), np.uint8)
+    for key in keys:
+        _, _, rid, cid, gpu = key
+        if rank is not None and int(gpu) != rank:
+            continue
+        kernel_causal = bool(causal) and isinstance(rid, (int, np.integer)) and isinstance(cid, (int, np.integer)) \
+            and int(rid) == int(cid)
+        for r in _ids(rid):
+            for c in _ids(cid):
+                if m[r, c] != EMPTY:
+                    raise ValueError(f"chunk ({r}, {c}) is covered by two kernels")
+                m[r, c] = CAUSAL if kernel_causal else FULL
+    return m
+
+
+def comp_kernels_from_schedule(schedule_table: np.ndarray, rank: Optional[int] = None) -> List[CompKey]:
+    """Keys in the reference's enumeration order (``search_algo/dependent_graph.py:235-240``):
+    batch, head, then row chunk k outer / column chunk l inner, every entry >= 0
+    (-1 = empty, ``search_algo/search_engine.py:363-370``)."""
+    st = np.asarray(schedule_table)
+    if st.ndim == 2:
+        st = st[None, None]
+    out = []
+    for i in range(st.shape[0]):
+        for j in range(st.shape[1]):
+            for k in range(st.shape[2]):
+                for l in range(st.shape[3]):
+                    g = int(st[i, j, k, l])
+                    if g >= 0 and (rank is None or g == rank):
+                        out.append((i, j, k, l, g))
+    return out
+
+
+class BlockSparseExecutor:
+    """Runs one device's share of a block-sparse attention on one GPU.
+
+    ``block_mask``: uint8 [row chunks, column chunks] of 0 EMPTY / 1 FULL / 2 CAUSAL for the
+    chunks this device computes; ``chunk`` = tokens per chunk (``S_per_partition``).
+    ``kernel_tiles`` > 1 splits the key range into that many kernel tiles whose partial
+    (O, LSE) are merged, as the streaming configuration does."""
+
+    def __init__(self, block_mask: np.ndarray, chunk: int, softmax_scale: Optional[float] = None,
+                 kernel_tiles: int = 1):
+        self.mask = np.ascontiguousarray(block_mask, dtype=np.uint8)
+        self.chunk = int(chunk)
+        self.softmax_scale = softmax_scale
+        self.tiles: TileList = build_tile_list(self.mask, block=self.chunk)
+        self.kernel_tiles: List[TileList] = []
+        if kernel_tiles > 1:
+            cols = np.nonzero(self.mask.any(0))[0]
+            for part in np.array_split(cols, min(kernel_tiles, max(1, len(cols)))):
+                sub = np.zeros_like(self.mask)
+                sub[:, part] = self.mask[:, part]
+                self.kernel_tiles.append(build_tile_list(sub, block=self.chunk))
+
+    @classmethod
+    def from_comp_kernels(cls, keys: Iterable[CompKey], n_row_chunks: int, n_col_chunks: int, chunk: int,
+                          causal: bool, rank: Optional[int] = None, **kw) -> "BlockSparseExecutor":
+        return cls(mask_from_comp_kernels(keys, n_row_chunks, n_col_chunks, causal, rank), chunk, **kw)
+
+    @classmethod
+    def from_schedule_table(cls, schedule_table: np.ndarray, block_table: np.ndarray, rank: int, chunk: int,
+                            **kw) -> "BlockSparseExecutor":
+        """``schedule_table[k, l] == rank`` selects this device's chunks; their types come from the
+        block table (``Block_Type`` values)."""
+        st = np.asarray(schedule_table)
+        st = st.reshape(st.shape[-2:])
+        return cls(np.where(st == rank, np.asarray(block_table, np.uint8), EMPTY).astype(np.uint8), chunk, **kw)
+
+    def forward(self, q, k, v, out=None, lse=None):
+        """-> (out, lse); one launch, or ``kernel_tiles`` launches + one merge."""
+        if not self.kernel_tiles:
+            return bsa_fwd(q, k, v, self.tiles, self.softmax_scale, out=out, lse=lse)
+        parts = [bsa_fwd(q, k, v, t, self.softmax_scale) for t in self.kernel_tiles]
+        return merge_partials([p[0] for p in parts], [p[1] for p in parts], out=out, lse=lse)
+
+    def backward(self, dout, q, k, v, out, lse, dq=None, dk=None, dv=None, softmax_d=None):
+        """-> (dq, dk, dv).  ``lse`` (and ``softmax_d``) are the rows' GLOBAL statistics: when this
+        device holds only part of a row's keys they are those of the merged result."""
+        if softmax_d is None:
+            softmax_d = softmax_delta(out, dout)
+        return bsa_bwd(dout, q, k, v, None, lse, self.tiles, self.softmax_scale, dq=dq, dk=dk, dv=dv,
+                       softmax_d=softmax_d)
+
+    @staticmethod
+    def reduce_fwd(parts: Sequence[Tuple[torch.Tensor, torch.Tensor]], out=None, lse=None):
+        """``Output_Row_Fwd.reduce`` for any number of partial (O, LSE) pairs."""
+        return merge_partials([p[0] for p in parts], [p[1] for p in parts], out=out, lse=lse)
+
+    @staticmethod
+    def reduce_bwd(parts: Sequence[torch.Tensor]) -> torch.Tensor:
+        """``Output_Row_Bwd.reduce`` / ``Output_Col_Bwd.reduce``: fp32 sum of partial gradients
+        (``ring_flash_attn/ring_flash_attn.py:110-118`` accumulates in fp32), returned in bf16."""
+        acc = parts[0].float()
+        for p in parts[1:]:
+            acc += p.float()
+        return acc.to(parts[0].dtype)
