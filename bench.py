@@ -27,7 +27,7 @@ FLOP_PER_CLK_PER_CU = 4096        # dense bf16 MFMA, CDNA4
 
 # HBM bytes per launch of the dominant kernel, from profiles/hbm_traffic_<workload>.txt
 # (rocprofv3 --pmc FETCH_SIZE x 2.0 + WRITE_SIZE x 1.0, scaling explained there).
-TRAFFIC_BYTES = {("c3", "dkdv_kernel"): 43.52e9, ("c5", "fwd_kernel"): 12.37e9}
+TRAFFIC_BYTES = {("c3", "dkdv_kernel"): 46.34e9, ("c5", "fwd_kernel"): 11.62e9}
 
 
 def log(*a):
@@ -214,6 +214,30 @@ def run_c5(steps, warmup):
             "fwd_plus_merge_tflops": F / wall_ms / 1e9}
 
 
+def run_mask_builder(name, steps):
+    """Device tile-list builder on one workload's block mask: 4 small launches (count, scan,
+    fill, order).  Bytes = block mask read + the eight tile-list arrays written."""
+    import torch
+    from ultraattn_amd.tilelist import build_tile_list, build_tile_list_device
+    mask = workload_mask(name)
+    host = build_tile_list(mask, BLOCK)
+    m = torch.from_numpy(mask.astype("uint8")).to("cuda:0")
+    dev = build_tile_list_device(m, BLOCK, nnz=host.nnz)
+    torch.cuda.synchronize()
+    same = all(bool((dev[n].cpu() == torch.from_numpy(getattr(host, n))).all())
+               for n in ("row_ptr", "col_idx", "flag", "col_ptr", "row_idx", "cflag", "q_order", "k_order"))
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(steps):
+        build_tile_list_device(m, BLOCK, nnz=host.nnz)
+    e1.record()
+    torch.cuda.synchronize()
+    ms = e0.elapsed_time(e1) / steps
+    nbytes = mask.size + 2 * host.nnz * 5 + 4 * (2 * (host.n_qtiles + host.n_ktiles) + 2)
+    return {"workload": name, "ms": ms, "bytes": nbytes, "gbps": nbytes / ms / 1e6, "nnz_tiles": host.nnz,
+            "matches_host_builder": same, "note": "latency-bound: 4 dependent launches over a few MB"}
+
+
 def probe_mfma(peak):
     """Sustained register-only MFMA rate with constant and with random operand bits."""
     import torch
@@ -347,6 +371,9 @@ def main():
                       "seq_kv": int(workload_mask(a.workload).shape[1]) * BLOCK},
            "frac_of_bf16_mfma_peak": value / peak, "peak_tflops": peak, "detail": main_res,
            "fwd_frac_of_peak": main_res["fwd_tflops"] / peak, "roofline": roof, "extra": extra}
+    if not a.no_extra:
+        out["mask_builder"] = run_mask_builder(a.workload if a.workload != "c5" else "c3", 20)
+        log(json.dumps(out["mask_builder"]))
     out["mfma_probe"] = probe_mfma(peak)
     log(json.dumps(out["mfma_probe"]))
     if not a.no_cpu:

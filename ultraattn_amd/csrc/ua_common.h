@@ -9,9 +9,7 @@ namespace ua {
 typedef __bf16 bf16;
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
 typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4;
-typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2;
 typedef __attribute__((ext_vector_type(16))) float f32x16;
-typedef __attribute__((ext_vector_type(8))) float f32x8;
 typedef __attribute__((ext_vector_type(4))) float f32x4;
 typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
 
@@ -64,20 +62,6 @@ __device__ __forceinline__ f32x16 mfma32(bf16x8 a, bf16x8 b, f32x16 c) {
   return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
 }
 
-// Copy one [128][128] bf16 tile from global memory into LDS with the layout `OFF`
-// (256 threads, 16 bytes per thread per pass, each pass covers 16 full rows).
-template <int (*OFF)(int, int)>
-__device__ __forceinline__ void stage_tile(unsigned char* smem, const bf16* g, int64_t row_stride, int tid) {
-  const int c = tid & 15, r0 = tid >> 4;
-  u32x4 val[8];
-#pragma unroll
-  for (int p = 0; p < 8; ++p)
-    val[p] = *reinterpret_cast<const u32x4*>(g + (int64_t)(p * 16 + r0) * row_stride + c * 8);
-#pragma unroll
-  for (int p = 0; p < 8; ++p)
-    *reinterpret_cast<u32x4*>(smem + OFF(p * 16 + r0, c)) = val[p];
-}
-
 // Per-lane constants of the transposing reads that build an A operand of X^T from a
 // row-major tile X[row][col] in LDS: the MFMA row index is the tile column
 // (32*mb + lane%32), the contraction index runs over tile rows.  For a 16-row step starting
@@ -100,39 +84,12 @@ __device__ __forceinline__ bf16x8 lds_read_tr_frag(const unsigned char* smem, co
   return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
 }
 
-// Asynchronous global -> LDS copy of 16 bytes per lane (global_load_lds_dwordx4): the wave's 64
-// lanes fill 1 KiB starting at the wave-uniform LDS address `lds_dst`, lane l at +16*l, each
-// from its own global address.  Completion is tracked by vmcnt.
-__device__ __forceinline__ void dma16(const bf16* gsrc, unsigned char* lds_dst) {
-  __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)gsrc,
-                                   (__attribute__((address_space(3))) void*)lds_dst, 16, 0, 0);
-}
 __device__ __forceinline__ void wait_vmem_all() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
 // Workgroup barrier that orders LDS traffic only: unlike __syncthreads() it does not wait for
 // the asynchronous global->LDS copies still in flight (they target another stage).
 __device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
 // Keeps a wave-uniform branch a branch (the optimiser may not turn its body into selects).
 __device__ __forceinline__ void keep_branch() { asm volatile("" ::: "memory"); }
-
-// Per-thread source offsets (in elements) for staging a [64][128] bf16 half tile (16 KiB) with
-// NW waves: each thread issues 16/NW DMA instructions; instruction i of wave w fills LDS rows
-// 4*(NW*i + w) .. +3; lane l lands in that group's row l/16, physical 16-byte slot l%16, so
-// it must fetch the logical chunk that the XOR layout `OFF` maps to that slot.
-template <int (*OFF)(int, int), int NW>
-__device__ __forceinline__ void dma_offsets(int (&off)[16 / NW], int64_t row_stride, int wave, int lane) {
-#pragma unroll
-  for (int i = 0; i < 16 / NW; ++i) {
-    const int r = 4 * (NW * i + wave) + (lane >> 4);
-    const int phys = lane & 15;
-    const int c = ((OFF(r, 0) - r * kRowBytes) >> 4) ^ phys;
-    off[i] = (int)(r * row_stride) + c * 8;
-  }
-}
-template <int NW>
-__device__ __forceinline__ void dma_half_tile(unsigned char* lds, const bf16* g, const int (&off)[16 / NW], int wave) {
-#pragma unroll
-  for (int i = 0; i < 16 / NW; ++i) dma16(g + off[i], lds + (NW * i + wave) * 1024);
-}
 
 // Wave-uniform reads of the (read-only) tile-list arrays through the scalar cache.
 __device__ __forceinline__ int32_t sload(const int32_t* p, int i) {
@@ -145,19 +102,21 @@ __device__ __forceinline__ int sload(const uint8_t* p, int i) {
   return (w >> (8 * (a & 3))) & 0xff;
 }
 
-// Buffer-addressed variant (buffer_load_dwordx4 ... lds): the source address is
-// descriptor base + per-lane byte offset `voff` + wave-uniform byte offset `soff`, so a tile's
-// address arithmetic stays on the scalar unit; reads beyond the descriptor's extent return 0.
+// Asynchronous global -> LDS copy (buffer_load_dwordx4 ... lds), 16 bytes per lane: the wave's
+// 64 lanes fill 1 KiB starting at the wave-uniform LDS address `lds_dst`, lane l at +16*l.  The
+// source address is descriptor base + per-lane byte offset `voff` + wave-uniform byte offset
+// `soff`, so a tile's address arithmetic stays on the scalar unit; reads beyond the descriptor's
+// extent return 0.  Completion is tracked by vmcnt.
 __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* base, uint32_t bytes) {
   return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, bytes, 0x00020000);
 }
 __device__ __forceinline__ void dma16_buf(__amdgpu_buffer_rsrc_t r, unsigned char* lds_dst, int voff, int soff) {
   __builtin_amdgcn_raw_ptr_buffer_load_lds(r, (__attribute__((address_space(3))) void*)lds_dst, 16, voff, soff, 0, 0);
 }
-__device__ __forceinline__ void dma4_buf(__amdgpu_buffer_rsrc_t r, unsigned char* lds_dst, int voff, int soff) {
-  __builtin_amdgcn_raw_ptr_buffer_load_lds(r, (__attribute__((address_space(3))) void*)lds_dst, 4, voff, soff, 0, 0);
-}
-// Per-thread byte offsets for staging a [64][128] bf16 half tile with NW waves (see dma_offsets).
+// Per-thread byte offsets for staging a [64][128] bf16 half tile (16 KiB) with NW waves: each
+// thread issues 16/NW copies; copy i of wave w fills LDS rows 4*(NW*i + w) .. +3; lane l lands in
+// that group's row l/16, physical 16-byte slot l%16, so it must fetch the logical chunk that the
+// XOR layout `OFF` maps to that slot.
 template <int (*OFF)(int, int), int NW>
 __device__ __forceinline__ void dma_voffsets(int (&off)[16 / NW], int row_stride, int wave, int lane) {
 #pragma unroll
