@@ -49,20 +49,50 @@ static int check_mask(const uint8_t* mask, int nqb, int nkb, int rate) {
 }
 
 // ---- device variant -----------------------------------------------------------------------
-// count: one thread per query tile (and per key tile) counts its active tiles.
-__global__ void tl_count_kernel(const uint8_t* mask, int nqb, int nkb, int rate, int32_t* qcnt, int32_t* kcnt) {
+// One wavefront per query tile (a "row" of the list) and per key tile (a "column"); lanes
+// stride over the blocks of that row or column of the block mask.  Number of active tiles
+// that block (qb, kb) gives to query tile qt = qb*rate + a: FULL rate, CAUSAL a + 1 (key
+// sub-tiles 0..a); to key tile kt = kb*rate + b: FULL rate, CAUSAL rate - b (query sub-tiles
+// b..rate-1).
+constexpr int kWavesPerGroup = 4;
+
+struct Line {          // one row or one column of the tile grid, as seen by its wavefront
+  bool is_row;
+  int id;              // tile index of the row or column
+  int n_blocks;        // blocks along it
+  int sub;             // id % rate
+  int64_t base, step;  // block (i) of the line sits at mask[base + i*step]
+};
+__device__ __forceinline__ bool line_of_wave(int nqb, int nkb, int rate, Line& ln) {
+  const int w = blockIdx.x * kWavesPerGroup + (threadIdx.x >> 6);
   const int nqt = nqb * rate, nkt = nkb * rate;
-  const int t = blockIdx.x * blockDim.x + threadIdx.x;
-  if (t < nqt) {
-    int n = 0;
-    for (int kt = 0; kt < nkt; ++kt) n += tile_type(mask, nkb, rate, t, kt) != 0;
-    qcnt[t] = n;
-  } else if (t < nqt + nkt) {
-    const int kt = t - nqt;
-    int n = 0;
-    for (int q = 0; q < nqt; ++q) n += tile_type(mask, nkb, rate, q, kt) != 0;
-    kcnt[kt] = n;
-  }
+  if (w >= nqt + nkt) return false;
+  ln.is_row = w < nqt;
+  ln.id = ln.is_row ? w : w - nqt;
+  ln.n_blocks = ln.is_row ? nkb : nqb;
+  ln.sub = ln.id % rate;
+  ln.base = ln.is_row ? (int64_t)(ln.id / rate) * nkb : ln.id / rate;
+  ln.step = ln.is_row ? 1 : nkb;
+  return true;
+}
+__device__ __forceinline__ int tiles_of_block(const Line& ln, int type, int rate) {
+  return type == 1 ? rate : (type == 2 ? (ln.is_row ? ln.sub + 1 : rate - ln.sub) : 0);
+}
+__device__ __forceinline__ int wave_sum(int v) {
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off);
+  return v;
+}
+
+__global__ __launch_bounds__(64 * kWavesPerGroup) void tl_count_kernel(const uint8_t* mask, int nqb, int nkb, int rate,
+                                                                        int32_t* qcnt, int32_t* kcnt) {
+  Line ln;
+  if (!line_of_wave(nqb, nkb, rate, ln)) return;
+  const int lane = threadIdx.x & 63;
+  int n = 0;
+  for (int i = lane; i < ln.n_blocks; i += 64) n += tiles_of_block(ln, mask[ln.base + i * ln.step], rate);
+  n = wave_sum(n);
+  if (lane == 0) (ln.is_row ? qcnt : kcnt)[ln.id] = n;
 }
 
 // scan: a single workgroup turns counts into exclusive prefix sums.
@@ -86,40 +116,60 @@ __global__ __launch_bounds__(1024) void tl_scan_kernel(const int32_t* cnt, int n
   if (tid == 1023) ptr[n] = part[1023];
 }
 
-// order: rank of a row = number of rows that precede it (one thread per row).
-__global__ void tl_order_kernel(const int32_t* qptr, const int32_t* qidx, int nq, int32_t* q_order,
-                                const int32_t* kptr, const int32_t* kidx, int nk, int32_t* k_order) {
-  const int t = blockIdx.x * blockDim.x + threadIdx.x;
+// fill: the wavefront walks its line 64 blocks at a time; an exclusive scan of the per-block
+// tile counts gives every lane the slot where its block's tiles go, in ascending tile order.
+__global__ __launch_bounds__(64 * kWavesPerGroup) void tl_fill_kernel(const uint8_t* mask, int nqb, int nkb, int rate,
+                                                                       const int32_t* row_ptr, int32_t* col_idx, uint8_t* flag,
+                                                                       const int32_t* col_ptr, int32_t* row_idx, uint8_t* cflag) {
+  Line ln;
+  if (!line_of_wave(nqb, nkb, rate, ln)) return;
+  const int lane = threadIdx.x & 63;
+  int32_t* idx = ln.is_row ? col_idx : row_idx;
+  uint8_t* flg = ln.is_row ? flag : cflag;
+  int e = (ln.is_row ? row_ptr : col_ptr)[ln.id];
+  for (int i0 = 0; i0 < ln.n_blocks; i0 += 64) {
+    const int i = i0 + lane;
+    const int type = i < ln.n_blocks ? mask[ln.base + i * ln.step] : 0;
+    const int c = tiles_of_block(ln, type, rate);
+    int incl = c;
+#pragma unroll
+    for (int off = 1; off < 64; off <<= 1) {
+      const int v = __shfl_up(incl, off);
+      if (lane >= off) incl += v;
+    }
+    int at = e + incl - c;
+    // sub-tiles along the line: a row takes key sub-tiles 0..sub of a causal block (the last one
+    // causal), a column takes query sub-tiles sub..rate-1 (the first one causal)
+    const int first = (type == 2 && !ln.is_row) ? ln.sub : 0;
+    for (int t = 0; t < c; ++t) {
+      const int s = first + t;
+      idx[at] = i * rate + s;
+      flg[at] = type == 2 && s == ln.sub;
+      ++at;
+    }
+    e += __shfl(incl, 63);
+  }
+}
+
+// order: rank of a line = number of lines that precede it; one workgroup per line, its threads
+// share the comparisons.
+__global__ __launch_bounds__(256) void tl_order_kernel(const int32_t* qptr, const int32_t* qidx, int nq, int32_t* q_order,
+                                                       const int32_t* kptr, const int32_t* kidx, int nk, int32_t* k_order) {
+  __shared__ int rank_s;
+  const int t = blockIdx.x;
   const int32_t* ptr = t < nq ? qptr : kptr;
   const int32_t* idx = t < nq ? qidx : kidx;
   const int n = t < nq ? nq : nk;
   int32_t* order = t < nq ? q_order : k_order;
   const int i = t < nq ? t : t - nq;
-  if (t >= nq + nk) return;
+  if (threadIdx.x == 0) rank_s = 0;
+  __syncthreads();
   int rank = 0;
-  for (int j = 0; j < n; ++j) rank += (j != i) && row_precedes(ptr, idx, n, j, i);
-  order[rank] = i;
-}
-
-__global__ void tl_fill_kernel(const uint8_t* mask, int nqb, int nkb, int rate,
-                               const int32_t* row_ptr, int32_t* col_idx, uint8_t* flag,
-                               const int32_t* col_ptr, int32_t* row_idx, uint8_t* cflag) {
-  const int nqt = nqb * rate, nkt = nkb * rate;
-  const int t = blockIdx.x * blockDim.x + threadIdx.x;
-  if (t < nqt) {
-    int e = row_ptr[t];
-    for (int kt = 0; kt < nkt; ++kt) {
-      const int ty = tile_type(mask, nkb, rate, t, kt);
-      if (ty) { col_idx[e] = kt; flag[e] = ty == 2; ++e; }
-    }
-  } else if (t < nqt + nkt) {
-    const int kt = t - nqt;
-    int e = col_ptr[kt];
-    for (int q = 0; q < nqt; ++q) {
-      const int ty = tile_type(mask, nkb, rate, q, kt);
-      if (ty) { row_idx[e] = q; cflag[e] = ty == 2; ++e; }
-    }
-  }
+  for (int j = threadIdx.x; j < n; j += 256) rank += (j != i) && row_precedes(ptr, idx, n, j, i);
+  rank = wave_sum(rank);
+  if ((threadIdx.x & 63) == 0) atomicAdd(&rank_s, rank);
+  __syncthreads();
+  if (threadIdx.x == 0) order[rank_s] = i;
 }
 
 }  // namespace ua
@@ -194,13 +244,13 @@ extern "C" int ua_tilelist_build_device(const uint8_t* block_mask, int n_qblocks
   hipStream_t st = (hipStream_t)stream;
   int32_t* qcnt = work;
   int32_t* kcnt = work + nqt + 1;
-  const int blocks = (nqt + nkt + 255) / 256;
-  hipLaunchKernelGGL(tl_count_kernel, dim3(blocks), dim3(256), 0, st, block_mask, n_qblocks, n_kblocks, rate, qcnt, kcnt);
+  const int blocks = (nqt + nkt + kWavesPerGroup - 1) / kWavesPerGroup;
+  hipLaunchKernelGGL(tl_count_kernel, dim3(blocks), dim3(64 * kWavesPerGroup), 0, st, block_mask, n_qblocks, n_kblocks, rate, qcnt, kcnt);
   hipLaunchKernelGGL(tl_scan_kernel, dim3(1), dim3(1024), 0, st, (const int32_t*)qcnt, nqt, row_ptr);
   hipLaunchKernelGGL(tl_scan_kernel, dim3(1), dim3(1024), 0, st, (const int32_t*)kcnt, nkt, col_ptr);
-  hipLaunchKernelGGL(tl_fill_kernel, dim3(blocks), dim3(256), 0, st, block_mask, n_qblocks, n_kblocks, rate,
+  hipLaunchKernelGGL(tl_fill_kernel, dim3(blocks), dim3(64 * kWavesPerGroup), 0, st, block_mask, n_qblocks, n_kblocks, rate,
                      (const int32_t*)row_ptr, col_idx, flag, (const int32_t*)col_ptr, row_idx, cflag);
-  hipLaunchKernelGGL(tl_order_kernel, dim3((nqt + nkt + 63) / 64), dim3(64), 0, st,
+  hipLaunchKernelGGL(tl_order_kernel, dim3(nqt + nkt), dim3(256), 0, st,
                      (const int32_t*)row_ptr, (const int32_t*)col_idx, nqt, q_order,
                      (const int32_t*)col_ptr, (const int32_t*)row_idx, nkt, k_order);
   return hipGetLastError() == hipSuccess ? UA_OK : UA_ERR_LAUNCH;
