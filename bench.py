@@ -238,6 +238,27 @@ def run_mask_builder(name, steps):
             "matches_host_builder": same, "note": "latency-bound: 4 dependent launches over a few MB"}
 
 
+def run_cols_gather(steps):
+    """Column gather of a fused rectangle at the 128k shape: 4 chunks of [K | V], 32768 keys each."""
+    import torch
+    from ultraattn_amd import packed
+    Y, ks = 4, (1, 32768, HEADS, 128)
+    n = 2 * Y * ks[1] * ks[2] * ks[3]
+    buf = torch.empty(n, dtype=torch.bfloat16, device="cuda:0").normal_()
+    out = torch.empty_like(buf)
+    packed.gather_cols(buf, Y, ks, out=out)
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(steps):
+        packed.gather_cols(buf, Y, ks, out=out)
+    e1.record()
+    torch.cuda.synchronize()
+    ms = e0.elapsed_time(e1) / steps
+    return {"ms": ms, "bytes": 4 * n, "gbps": 4 * n / ms / 1e6, "frac_of_hbm": 4 * n / ms / 1e6 / HBM_PEAK_GBPS,
+            "shape": "[4, 2, 1, 32768, 32, 128] -> [2, 1, 131072, 32, 128] bf16, read + write"}
+
+
 def probe_mfma(peak):
     """Sustained register-only MFMA rate with constant and with random operand bits."""
     import torch
@@ -374,6 +395,8 @@ def main():
     if not a.no_extra:
         out["mask_builder"] = run_mask_builder(a.workload if a.workload != "c5" else "c3", 20)
         log(json.dumps(out["mask_builder"]))
+        out["cols_gather"] = run_cols_gather(10)
+        log(json.dumps(out["cols_gather"]))
     out["mfma_probe"] = probe_mfma(peak)
     log(json.dumps(out["mfma_probe"]))
     if not a.no_cpu:

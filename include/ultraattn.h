@@ -130,6 +130,21 @@ int ua_bsa_bwd_dq(const void *q, const void *k, const void *v, const void *dout,
 int ua_merge(const void *const *o_parts, const float *const *lse_parts, int n_parts,
              void *o, float *lse, int batch, int seqlen, int n_heads, int head_dim, void *stream);
 
+/* ---- column-buffer layout changes around a fused rectangle -----------------------------------
+ * Replace the two torch transpose+contiguous copies of the X x Y path:
+ *   ua_cols_gather : buf.view(Y,2,B,Skv,Nh,D).transpose(0,1).transpose(1,2).flatten(2,3).contiguous()
+ *                    (orchestrated_attn/orchestrated_attn_impl.py:269 forward, :512 backward):
+ *                    src [n_chunks, 2, batch, inner] -> dst [2, batch, n_chunks, inner], so that
+ *                    dst is one K and one V of n_chunks*Skv keys each;
+ *   ua_cols_scatter: oc.view(2, Y, K_nelem).transpose(0,1).contiguous()
+ *                    (orchestrated_attn_impl.py:548): src [2, batch, n_chunks, inner] ->
+ *                    dst [n_chunks, 2, batch, inner], [dK | dV] of the rectangle back to per-chunk
+ *                    [dK | dV] (the reference has batch = 1 there).
+ * inner_elems = Skv*Nh*D bf16 elements, a multiple of 8; src and dst are device pointers, 16-byte
+ * aligned, and must not overlap; 2*n_chunks*batch <= 65535.                                      */
+int ua_cols_gather(const void *src, void *dst, int n_chunks, int batch, int64_t inner_elems, void *stream);
+int ua_cols_scatter(const void *src, void *dst, int n_chunks, int batch, int64_t inner_elems, void *stream);
+
 /* ---- diagnostic (no counterpart in the reference) ----------------------------------------------
  * Runs n_blocks workgroups of 256 threads, each wave issuing 4 * iters register-only
  * v_mfma_f32_32x32x16_bf16 (32768 flop each) on the 512 x 16 bytes of operand bits at `operands`

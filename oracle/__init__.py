@@ -16,7 +16,9 @@ its root):
   the reference itself uses as its check (``easy_context/dist_flash_attn/lightseq_async_attn.py:482-488``);
 * the merge follows ``ring_flash_attn/utils.py:38-52, 78-99`` line by line;
 * the block-mask algebra follows ``search_algo/bsa_config.py:177-213`` and the tile
-  enumeration order follows ``search_algo/dependent_graph.py:235-240``.
+  enumeration order follows ``search_algo/dependent_graph.py:235-240``;
+* the column-buffer gather / scatter around a fused rectangle follows
+  ``orchestrated_attn/orchestrated_attn_impl.py:269, 512, 548``.
 
 Pinning status (what each function is checked against, see tests/test_oracle_*.py):
 
@@ -28,6 +30,8 @@ Pinning status (what each function is checked against, see tests/test_oracle_*.p
                         union of key sets, equal-LSE average, -inf identity.          PINNED
 * ``tilelist``        : brute-force element mask, counts derived independently,
                         reference-held mask strings and allocation logs.              PINNED
+* ``layout_oracle``   : explicit index loops, the reference's torch view/transpose chain,
+                        round trip.                                                   PINNED
 * flash_attn fork's own numerics (rounding order inside its CUDA kernel): no reference
   test or fixture pins a number at that boundary                                      PARITY UNPINNED
 """

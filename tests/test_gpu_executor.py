@@ -9,7 +9,7 @@ import torch
 
 from oracle import attn_oracle as ao
 from tests.gpu_util import ATOL_O, RTOL_LSE, SCALE, lse_rel_err, max_abs, oracle_fwd_bwd, seeded_inputs
-from ultraattn_amd import masks, packed
+from ultraattn_amd import masks, ops, packed
 from ultraattn_amd.executor import BlockSparseExecutor, comp_kernels_from_schedule
 
 pytestmark = pytest.mark.gpu
@@ -88,3 +88,50 @@ def test_kernels_run_in_place_on_packed_buffers():
     g2 = packed.OutputRowBwd(gq.data.clone(), qs)
     gq.reduce(g2)
     assert max_abs(gq.dQ, 2 * rq) <= 2 * ATOL_O
+
+
+@pytest.mark.parametrize("Y,ks", [(2, (1, 128, 2, 128)), (3, (2, 40, 3, 8)), (1, (1, 8, 1, 8)), (4, (1, 2048, 8, 128))])
+def test_column_gather_and_scatter_are_bit_exact(Y, ks):
+    from oracle import layout_oracle as lo
+    B, S, Nh, D = ks
+    n = 2 * Y * B * S * Nh * D
+    g = torch.Generator().manual_seed(Y)
+    raw = torch.randint(-2 ** 15, 2 ** 15, (n,), generator=g, dtype=torch.int16)
+    buf = raw.view(torch.bfloat16).to(DEV)
+    col = packed.gather_cols(buf, Y, ks)
+    want = lo.cols_gather(raw.numpy(), Y, ks)
+    assert col.K.shape == (B, Y * S, Nh, D)
+    assert np.array_equal(col.K.cpu().view(torch.int16).numpy(), want[0])
+    assert np.array_equal(col.V.cpu().view(torch.int16).numpy(), want[1])
+    back = packed.scatter_cols(packed.OutputColBwd(col.data, (B, Y * S, Nh, D)), Y, ks)
+    assert np.array_equal(back.cpu().view(torch.int16).numpy(), raw.numpy())
+    want_s = lo.cols_scatter(raw.numpy(), Y, ks).reshape(-1)
+    got_s = packed.scatter_cols(packed.OutputColBwd(buf, (B, Y * S, Nh, D)), Y, ks)
+    assert np.array_equal(got_s.cpu().view(torch.int16).numpy(), want_s)
+
+
+def test_column_gather_rejects_bad_arguments():
+    buf = torch.zeros(4096, dtype=torch.bfloat16, device=DEV)
+    with pytest.raises(RuntimeError):       # inner not a multiple of 8 elements
+        packed.gather_cols(buf, 2, (1, 3, 1, 4))
+    with pytest.raises(RuntimeError):       # source and destination overlap
+        packed.gather_cols(buf, 2, (1, 8, 1, 8), out=buf[8:])
+    with pytest.raises(ValueError):         # buffer too small
+        packed.gather_cols(buf, 2, (1, 128, 2, 128))
+
+
+def test_fused_rectangle_reads_gathered_columns():
+    """Y received column chunks -> gather -> one forward launch over Y*Skv keys equals the oracle on
+    the concatenated keys (the X x Y step of orchestrated_attn_impl.py:255-279)."""
+    Y, Nh, S = 3, 2, 256
+    g = torch.Generator().manual_seed(5)
+    q = torch.randn(1, S, Nh, 128, generator=g).to(torch.bfloat16)
+    chunks = [torch.randn(2, 1, S, Nh, 128, generator=g).to(torch.bfloat16) for _ in range(Y)]
+    buf = torch.stack(chunks).reshape(-1).to(DEV)
+    col = packed.gather_cols(buf, Y, (1, S, Nh, 128))
+    mask = np.ones((1, Y), np.uint8)
+    o, lse = ops.bsa_fwd(q.to(DEV), col.K, col.V, mask, SCALE, block=S)
+    k = torch.cat([c[0] for c in chunks], dim=1)
+    v = torch.cat([c[1] for c in chunks], dim=1)
+    ro, rl = ao.dense_fwd(q, k, v, SCALE, ao.element_mask(mask, S))
+    assert max_abs(o, ro) <= ATOL_O and lse_rel_err(lse, rl) <= RTOL_LSE

@@ -24,6 +24,8 @@ SIGNATURES = {
     "ua_probe_mfma": (c_int, [c_void_p, c_void_p, c_int, c_int, c_void_p]),
     "ua_merge": (c_int, [POINTER(c_void_p), POINTER(c_void_p), c_int, c_void_p, c_void_p,
                          c_int, c_int, c_int, c_int, c_void_p]),
+    "ua_cols_gather": (c_int, [c_void_p, c_void_p, c_int, c_int, c_int64, c_void_p]),
+    "ua_cols_scatter": (c_int, [c_void_p, c_void_p, c_int, c_int, c_int64, c_void_p]),
 }
 
 _lib = None

@@ -9,7 +9,7 @@ PKG_DIR = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(PKG_DIR, "csrc")
 LIB_NAME = "libultraattn_hip.so"
 LIB_PATH = os.path.join(PKG_DIR, LIB_NAME)
-SOURCES = ["api.hip", "tilelist.hip", "merge.hip", "fwd.hip", "bwd.hip", "probe.hip"]
+SOURCES = ["api.hip", "tilelist.hip", "merge.hip", "glue.hip", "fwd.hip", "bwd.hip", "probe.hip"]
 # -packed-fp32-ops: keep the compiler from forming v_pk_{add,mul,fma}_f32 out of scalar code.
 HIPCC_FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-Wall", "-Wno-unused-result",
                "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]

@@ -1,0 +1,78 @@
+// Column-buffer layout changes around a fused rectangle of Y column chunks.
+//
+// A received column buffer is Y chunks of [K | V]: [Y, 2, B, inner] with inner = Skv*Nh*D
+// contiguous bf16.  The kernels want one K and one V over all Y*Skv keys: [2, B, Y, inner].
+// The inverse takes [dK | dV] of the fused rectangle back to per-chunk [dK | dV].  Both are a
+// permutation of 2*B*Y contiguous chunks: one HBM-bound copy kernel, 16 bytes per lane,
+// streamed past the caches (every byte is touched once).
+#include <algorithm>
+#include "ua_common.h"
+
+namespace ua {
+
+constexpr int kCopyThreads = 256;
+constexpr int kCopyVecs = 4;                                   // 16-byte vectors per thread and step
+constexpr int kTargetGroups = 4096;                            // workgroups per launch, 16 per CU
+constexpr int64_t kSegBytes = (int64_t)kCopyThreads * kCopyVecs * 16;   // per workgroup and step
+
+struct PermuteParams {
+  const unsigned char* src;
+  unsigned char* dst;
+  int64_t chunk_bytes;
+  int n_y, n_b;
+  int gather;          // 1: src [Y,2,B] -> dst [2,B,Y];  0: src [2,B,Y] -> dst [Y,2,B]
+};
+
+__global__ __launch_bounds__(kCopyThreads) void permute_chunks_kernel(PermuteParams p) {
+  // blockIdx.y walks the chunks in [2,B,Y] order (the order of the side that is not [Y,2,B])
+  const int id = blockIdx.y;
+  const int y = id % p.n_y, b = (id / p.n_y) % p.n_b, c = id / (p.n_y * p.n_b);
+  const int64_t fused = id, split = ((int64_t)y * 2 + c) * p.n_b + b;
+  const unsigned char* s = p.src + (p.gather ? split : fused) * p.chunk_bytes;
+  unsigned char* d = p.dst + (p.gather ? fused : split) * p.chunk_bytes;
+  // a workgroup walks its chunk in strides of the grid's width: few, long-lived workgroups keep
+  // more loads in flight than one short workgroup per segment
+  for (int64_t seg0 = (int64_t)blockIdx.x * kSegBytes; seg0 < p.chunk_bytes; seg0 += (int64_t)gridDim.x * kSegBytes) {
+    u32x4 v[kCopyVecs];
+#pragma unroll
+    for (int i = 0; i < kCopyVecs; ++i) {
+      const int64_t off = seg0 + ((int64_t)i * kCopyThreads + threadIdx.x) * 16;
+      if (off < p.chunk_bytes) v[i] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(s + off));
+    }
+#pragma unroll
+    for (int i = 0; i < kCopyVecs; ++i) {
+      const int64_t off = seg0 + ((int64_t)i * kCopyThreads + threadIdx.x) * 16;
+      if (off < p.chunk_bytes) __builtin_nontemporal_store(v[i], reinterpret_cast<u32x4*>(d + off));
+    }
+  }
+}
+
+static int launch_permute(const void* src, void* dst, int n_chunks, int batch, int64_t inner_elems, int gather, void* stream) {
+  if (!src || !dst) return UA_ERR_NULL;
+  if (n_chunks <= 0 || batch <= 0 || inner_elems <= 0) return UA_ERR_SHAPE;
+  if ((int64_t)2 * n_chunks * batch > 65535) return UA_ERR_SHAPE;          // grid y
+  if (inner_elems % 8 != 0 || !aligned16(src) || !aligned16(dst)) return UA_ERR_ALIGN;
+  const int64_t total = (int64_t)2 * n_chunks * batch * inner_elems * 2;
+  const unsigned char* s = (const unsigned char*)src;
+  const unsigned char* d = (const unsigned char*)dst;
+  if (s < d + total && d < s + total) return UA_ERR_SHAPE;                  // no in-place permutation
+  if (int rc = check_device()) return rc;
+  PermuteParams p;
+  p.src = s; p.dst = (unsigned char*)dst; p.chunk_bytes = inner_elems * 2; p.n_y = n_chunks; p.n_b = batch; p.gather = gather;
+  const int64_t segs = (p.chunk_bytes + kSegBytes - 1) / kSegBytes;
+  const int lines = 2 * n_chunks * batch;
+  const int64_t width = std::min<int64_t>(segs, std::max<int64_t>(1, kTargetGroups / lines));
+  hipLaunchKernelGGL(permute_chunks_kernel, dim3((unsigned)width, lines), dim3(kCopyThreads), 0,
+                     (hipStream_t)stream, p);
+  return hipGetLastError() == hipSuccess ? UA_OK : UA_ERR_LAUNCH;
+}
+
+}  // namespace ua
+
+extern "C" int ua_cols_gather(const void* src, void* dst, int n_chunks, int batch, int64_t inner_elems, void* stream) {
+  return ua::launch_permute(src, dst, n_chunks, batch, inner_elems, 1, stream);
+}
+
+extern "C" int ua_cols_scatter(const void* src, void* dst, int n_chunks, int batch, int64_t inner_elems, void* stream) {
+  return ua::launch_permute(src, dst, n_chunks, batch, inner_elems, 0, stream);
+}

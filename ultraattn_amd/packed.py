@@ -127,3 +127,42 @@ class OutputColBwd:
 
     def reduce(self, other: "OutputColBwd") -> None:
         self.data.add_(other.data)
+
+
+def _permute_cols(entry: str, src: torch.Tensor, n_chunks: int, k_shape, out: torch.Tensor = None) -> torch.Tensor:
+    from . import _lib
+    B, S, Nh, D = k_shape
+    inner = S * Nh * D
+    n = 2 * n_chunks * B * inner
+    if src.dim() != 1 or src.dtype != torch.bfloat16 or not src.is_cuda or src.numel() < n:
+        raise ValueError(f"the column buffer must be a flat bfloat16 CUDA tensor of at least {n} elements")
+    out = torch.empty(n, dtype=torch.bfloat16, device=src.device) if out is None else out
+    if out.dim() != 1 or out.dtype != torch.bfloat16 or out.device != src.device or out.numel() < n:
+        raise ValueError(f"out must be a flat bfloat16 tensor of at least {n} elements on the source's device")
+    lib = _lib.load()
+    with torch.cuda.device(src.device):
+        st = torch.cuda.current_stream().cuda_stream
+        rc = getattr(lib, entry)(src.data_ptr(), out.data_ptr(), n_chunks, B, inner, st)
+    _lib.check(rc, entry)
+    return out
+
+
+def gather_cols(buf: torch.Tensor, n_chunks: int, k_shape, out: torch.Tensor = None) -> InputColFwd:
+    """Fused-rectangle column input: ``buf`` holds ``n_chunks`` received column chunks, each
+    ``[K | V]`` of shape ``k_shape`` (B, Skv, Nh, D): ``[Y, 2, B, Skv, Nh, D]``.  Returns the
+    ``InputColFwd`` over ``[2, B, Y*Skv, Nh, D]`` — one K and one V across all chunks — produced
+    by one HBM-bound copy kernel in place of
+    ``view(Y,2,B,Skv,Nh,D).transpose(0,1).transpose(1,2).flatten(2,3).contiguous()``
+    (``orchestrated_attn/orchestrated_attn_impl.py:269, 512``)."""
+    B, S, Nh, D = k_shape
+    data = _permute_cols("ua_cols_gather", buf, n_chunks, k_shape, out)
+    return InputColFwd(data, (B, n_chunks * S, Nh, D))
+
+
+def scatter_cols(col_out: OutputColBwd, n_chunks: int, k_shape, out: torch.Tensor = None) -> torch.Tensor:
+    """Inverse for the column output of a fused rectangle: ``col_out.data`` is ``[dK | dV]`` over
+    ``Y*Skv`` keys (``[2, B, Y*Skv, Nh, D]``); returns the flat ``[Y, 2, B, Skv, Nh, D]`` buffer
+    of per-chunk ``[dK | dV]`` that the column reduce-scatter sends
+    (``oc.view(2, Y, K_nelem).transpose(0,1).contiguous()``,
+    ``orchestrated_attn/orchestrated_attn_impl.py:548``)."""
+    return _permute_cols("ua_cols_scatter", col_out.data, n_chunks, k_shape, out)
