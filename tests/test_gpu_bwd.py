@@ -46,6 +46,9 @@ CASES = {
     "batch2_heads5": (lambda: masks.config_causal(3), 128, 5, 2),
     "single_causal_tile": (lambda: np.full((1, 1), 2, np.uint8), 128, 1, 1),
     "rect_6x1": (lambda: np.ones((6, 1), np.uint8), 128, 2, 1),
+    # every XCD owns whole heads; 3 / 5 / 6 tile rows and columns leave the last dispatch team short
+    "heads16_rows3_cols5": (lambda: np.random.RandomState(1).randint(0, 2, size=(3, 5)).astype(np.uint8), 128, 16, 1),
+    "heads8_batch2_rows6": (lambda: masks.config_causal(3), 256, 8, 2),
 }
 
 

@@ -45,6 +45,11 @@ CASES = {
     "rect_1x6": (lambda: np.ones((1, 6), np.uint8), 128, 2, 1),
     "canonical_stride": (lambda: masks.canonical_block_table(0), 128, 2, 1),
     "canonical_stream": (lambda: masks.canonical_block_table(3), 256, 2, 1),
+    # 16 and 8 (batch, head) pairs: every XCD owns whole heads; 3 / 5 / 6 tile rows and columns do
+    # not fill the last dispatch team
+    "heads16_rows3_cols5": (lambda: np.random.RandomState(1).randint(0, 2, size=(3, 5)).astype(np.uint8), 128, 16, 1),
+    "heads8_batch2_rows6": (lambda: masks.config_causal(3), 256, 8, 2),
+    "heads8_rows5": (lambda: masks.config_causal(5), 128, 8, 1),
 }
 
 

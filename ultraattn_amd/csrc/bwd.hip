@@ -316,7 +316,7 @@ __global__ __launch_bounds__(512) void dkdv_kernel(const BwdParams p) {
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave8 = __builtin_amdgcn_readfirstlane(tid >> 6);      // 0..7
   int pos, bh;
-  map_block(blockIdx.x, p.batch * p.n_heads, p.heads_per_xcd, pos, bh);
+  map_block(blockIdx.x, p.batch * p.n_heads, p.heads_per_xcd, p.n_ktiles, pos, bh);
   const int kt = sload(p.order, pos);
   const int b = bh / p.n_heads, h = bh % p.n_heads;
   const DkdvStage stg[2] = {{sQ0, sdO0, sStat0}, {sQ1, sdO1, sStat1}};
@@ -393,7 +393,7 @@ __global__ __launch_bounds__(256, 2) void dq_kernel(const BwdParams p) {
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int l32 = lane & 31, hi = lane >> 5;
   int pos, bh;
-  map_block(blockIdx.x, p.batch * p.n_heads, p.heads_per_xcd, pos, bh);
+  map_block(blockIdx.x, p.batch * p.n_heads, p.heads_per_xcd, p.n_qtiles, pos, bh);
   const int qt = sload(p.order, pos);
   const int b = bh / p.n_heads, h = bh % p.n_heads;
   const int64_t seq_q = (int64_t)p.n_qtiles * kTile;

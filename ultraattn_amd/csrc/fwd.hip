@@ -142,7 +142,7 @@ __global__ __launch_bounds__(256, 2) void fwd_kernel(const FwdParams p) {
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int l32 = lane & 31, hi = lane >> 5;
   int pos, bh;
-  map_block(blockIdx.x, p.batch * p.n_heads, p.heads_per_xcd, pos, bh);
+  map_block(blockIdx.x, p.batch * p.n_heads, p.heads_per_xcd, p.n_qtiles, pos, bh);
   const int qt = sload(p.q_order, pos);
   const int b = bh / p.n_heads, h = bh % p.n_heads;
 

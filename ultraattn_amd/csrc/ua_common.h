@@ -134,13 +134,32 @@ __device__ __forceinline__ void dma_half_tile_buf(unsigned char* lds, __amdgpu_b
 }
 
 // blockIdx -> (position in the launch order, batch*head).  Consecutive workgroups go to
-// consecutive XCDs; each XCD gets its own heads so that tiles which share operands meet in
-// one L2.  heads_per_xcd = batch*n_heads/8 when divisible, else 0 (plain mapping).
-__device__ __forceinline__ void map_block(int bid, int nbh, int heads_per_xcd, int& pos, int& bh) {
+// consecutive XCDs.  Each XCD gets its own heads (heads_per_xcd = batch*n_heads/8 when
+// divisible, else 0 = plain mapping) and works on them kHeadGroup at a time, so that the
+// workgroups resident on an XCD belong to few heads and share K/V (or Q/dO) tiles in its L2.
+// Within a head group the dispatch order goes team by team: a team is kTeam consecutive
+// positions of the launch order (rows with the same or nearly the same tile lists); its
+// members are dispatched back to back, start together and walk their lists in step.
+constexpr int kHeadGroup = 2;
+constexpr int kTeam = 4;
+__device__ __forceinline__ void map_block(int bid, int nbh, int heads_per_xcd, int n_pos, int& pos, int& bh) {
   if (heads_per_xcd > 0) {
     const int xcd = bid & 7, idx = bid >> 3;
-    pos = idx / heads_per_xcd;
-    bh = xcd * heads_per_xcd + idx % heads_per_xcd;
+    const int g = (heads_per_xcd % kHeadGroup == 0) ? kHeadGroup : 1;
+    const int per_group = n_pos * g;
+    const int hg = idx / per_group, r = idx % per_group;
+    const int full = (n_pos / kTeam) * kTeam;        // positions in complete teams
+    int hs;
+    if (r < full * g) {
+      const int team = r / (kTeam * g), rr = r % (kTeam * g);
+      hs = rr / kTeam;
+      pos = team * kTeam + rr % kTeam;
+    } else {                                         // the last, shorter team
+      const int t = n_pos - full, rr = r - full * g;
+      hs = rr / t;
+      pos = full + rr % t;
+    }
+    bh = xcd * heads_per_xcd + hg * g + hs;
   } else {
     pos = bid / nbh;
     bh = bid % nbh;
