@@ -259,6 +259,100 @@ def run_cols_gather(steps):
             "shape": "[4, 2, 1, 32768, 32, 128] -> [2, 1, 131072, 32, 128] bf16, read + write"}
 
 
+class PowerSampler:
+    """Samples the socket power and the shader clock with `amd-smi metric -p -c` from a host thread
+    while the GPU works (nothing is sampled inside the timed step loop of the benchmark)."""
+
+    def __init__(self):
+        import shutil
+        self.exe = shutil.which("amd-smi")
+        self.samples = []
+        self._stop = False
+
+    def _poll(self):
+        import subprocess
+        while not self._stop:
+            try:
+                out = subprocess.run([self.exe, "metric", "-p", "-c"], capture_output=True, text=True, timeout=5).stdout
+            except Exception:
+                break
+            watts = mhz = None
+            section = ""
+            for line in out.splitlines():
+                t = line.strip()
+                if t.endswith(":"):
+                    section = t
+                if t.startswith("SOCKET_POWER:"):
+                    watts = t.split()[1]
+                if section.startswith("GFX_0") and t.startswith("CLK:"):
+                    mhz = t.split()[1]
+            try:
+                self.samples.append((float(watts), float(mhz)))
+            except (TypeError, ValueError):
+                pass
+            time.sleep(0.1)
+
+    def measure(self, fn, seconds, sync):
+        """Runs fn() repeatedly for `seconds`; returns median power / clock over the samples taken
+        after the first third of the interval, or None without amd-smi."""
+        import threading
+        if not self.exe:
+            return None
+        self.samples, self._stop = [], False
+        th = threading.Thread(target=self._poll)
+        th.start()
+        t0 = time.perf_counter()
+        while time.perf_counter() - t0 < seconds:
+            for _ in range(3):
+                fn()
+            sync()
+        self._stop = True
+        th.join()
+        keep = self.samples[len(self.samples) // 3:]
+        if not keep:
+            return None
+        med = lambda xs: sorted(xs)[len(xs) // 2]
+        return {"socket_power_w": med([w for w, _ in keep]), "gfx_clock_mhz": med([c for _, c in keep]), "samples": len(keep)}
+
+
+def run_power(name):
+    """Socket power and shader clock while each kernel of the workload runs back to back, next to a
+    register-only MFMA loop and a plain copy: shows which kernels sit at the board's power limit."""
+    import torch
+    from ultraattn_amd import _lib, ops
+    from ultraattn_amd.tilelist import build_tile_list
+    dev = "cuda:0"
+    sampler = PowerSampler()
+    if not sampler.exe:
+        return None
+    mask = workload_mask(name)
+    g = torch.Generator(device=dev).manual_seed(0)
+    mk = lambda n: torch.randn(1, n * BLOCK, HEADS, 128, device=dev, dtype=torch.float32, generator=g).to(torch.bfloat16)
+    q, k, v, do = mk(mask.shape[0]), mk(mask.shape[1]), mk(mask.shape[1]), mk(mask.shape[0])
+    tl = build_tile_list(mask, BLOCK)
+    o, lse = ops.bsa_fwd(q, k, v, tl, SCALE)
+    delta = ops.softmax_delta(o, do)
+    dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+    lib = _lib.load()
+    st = torch.cuda.current_stream().cuda_stream
+    rnd = torch.randn(512 * 8, device=dev).to(torch.bfloat16)
+    one = torch.ones(512 * 8, dtype=torch.bfloat16, device=dev)
+    sink = torch.empty(512 * 256, dtype=torch.float32, device=dev)
+    src = torch.empty(1 << 30, dtype=torch.uint8, device=dev)
+    dst = torch.empty_like(src)
+    runs = {
+        "forward": lambda: ops.bsa_fwd(q, k, v, tl, SCALE, out=o, lse=lse),
+        "backward": lambda: ops.bsa_bwd(do, q, k, v, None, lse, tl, SCALE, dq=dq, dk=dk, dv=dv, softmax_d=delta),
+        "mfma_random_operands": lambda: lib.ua_probe_mfma(rnd.data_ptr(), sink.data_ptr(), 512, 20000, st),
+        "mfma_constant_operands": lambda: lib.ua_probe_mfma(one.data_ptr(), sink.data_ptr(), 512, 20000, st),
+        "copy_1GiB": lambda: dst.copy_(src),
+    }
+    out = {"workload": name}
+    for key, fn in runs.items():
+        out[key] = sampler.measure(fn, 1.5, torch.cuda.synchronize)
+    return out
+
+
 def probe_mfma(peak):
     """Sustained register-only MFMA rate with constant and with random operand bits."""
     import torch
@@ -397,6 +491,10 @@ def main():
         log(json.dumps(out["mask_builder"]))
         out["cols_gather"] = run_cols_gather(10)
         log(json.dumps(out["cols_gather"]))
+        if a.workload != "c5":
+            torch.cuda.empty_cache()
+            out["power"] = run_power(a.workload)
+            log(json.dumps(out["power"]))
     out["mfma_probe"] = probe_mfma(peak)
     log(json.dumps(out["mfma_probe"]))
     if not a.no_cpu:
