@@ -16,6 +16,7 @@
 //                Here a lane holds one query column, so lse and delta are per-lane scalars.
 //  P = exp2(scale*log2e*S - lse*log2e);  dS = P * (dP - delta);  dQ, dK are scaled by
 //  softmax_scale on output.
+#include <type_traits>
 #include "ua_common.h"
 
 namespace ua {
@@ -77,68 +78,120 @@ __device__ __forceinline__ bf16x8 read_tr_pair(const unsigned char* smem, int of
 
 // ---- dK/dV ------------------------------------------------------------------------------------
 // The workgroup has 8 wavefronts in two groups of 4; wave w of either group owns key rows
-// 32w..32w+31 of the key tile, and each SIMD hosts one wave of each group.  Per block of 32
-// query rows:
-//   group A:  S = Q K^T -> P = exp2(..) -> hands P (bf16) to its partner through LDS;  dV^T += dO^T P
-//   group B:  dP = dO V^T;  takes P;  dS = P * (dP - delta);                             dK^T += Q^T dS
-// Both groups issue 16 MFMAs per block and about the same vector work, fit in 256 registers
-// (two waves per SIMD, accumulators in VGPRs), and one group's MFMAs overlap the other's exp2 /
-// pointwise work.
+// 32w..32w+31 of the key tile, and each SIMD hosts one wave of each group.  Work is handed out
+// in half tiles of 64 query rows (two blocks of 32):
+//   group A, half tile i  :  S = Q K^T -> P = exp2(..), left in LDS for its partner;  dV^T += dO^T P
+//   group B, half tile i-1:  dS = P * dP' (dP' = dO V^T - delta, kept from the step before);
+//                            dK^T += Q^T dS;   then dP' of half tile i for the next step
+// Group B thus runs one half tile behind group A, nothing inside a step depends on the other
+// group, and one workgroup barrier per half tile is the only synchronisation.  Both groups issue
+// 32 MFMAs per step; A's order is MFMA, vector, MFMA and B's is vector, MFMA, MFMA, so one
+// group's MFMAs cover the other's exp2 / pointwise work.
+//
+// Q / dO half tiles, P and the rows' statistics live in rings of three stages inside one LDS
+// array: copies into stage i+1 are in flight while A reads stage i and B reads stage i-1.  All
+// LDS accesses use absolute addresses = one per-lane register + a compile-time constant that
+// names ring and stage (it fits the instructions' 16-bit offset field), so the three stages cost
+// no extra address registers.  The asynchronous copies are issued from inline assembly: the
+// compiler then does not order the LDS reads of other stages behind them; completion is awaited
+// explicitly (s_waitcnt vmcnt(0)) before the barrier that ends the step.
+#define UA_LDS __attribute__((address_space(3)))
 constexpr int kPBlockBytes = 4 * 2048;      // P of one 32-row block: 4 waves x (64 lanes x 32 B)
+constexpr int kPHalfBytes = 2 * kPBlockBytes;
+constexpr int kStatBytes = 2 * kHalf * 4;   // -lse/scale and -delta of one half tile
+constexpr int kRingQ = 0, kRingDO = 3 * kHalfBytes, kRingP = 6 * kHalfBytes, kRingStat = kRingP + 3 * kPHalfBytes;
+constexpr int kDkdvLdsBytes = kRingStat + 3 * kStatBytes;
+static_assert(2 * kHalfBytes + kHalfBytes / 2 + 16 * kRowBytes + 8 * kRowBytes + 256 < 65536, "stage constants fit the offset field");
 
-// Eight transposed fragments (2 steps of 16 rows x 4 d-blocks) feeding acc[mbd] += X^T * bfrag[t],
-// fetched kAhead fragments ahead of the MFMA that consumes them.
-__device__ __forceinline__ void mfma_tr_block(const unsigned char* sX, const LaneOffsU& lo, int blk,
-                                              const bf16x8 (&bfrag)[2], f32x16 (&acc)[4]) {
-  constexpr int kAhead = 3;
-  bf16x8 fr[8];
+__device__ __forceinline__ void keep_in_register(uint32_t& x) { asm volatile("" : "+v"(x)); }
+__device__ __forceinline__ bf16x8 lds_abs_b128(uint32_t a) { return *reinterpret_cast<const UA_LDS bf16x8*>(a); }
+__device__ __forceinline__ bf16x8 lds_abs_tr_pair(uint32_t a_lo, uint32_t a_hi) {
+  const bf16x4 x = __builtin_amdgcn_ds_read_tr16_b64_v4bf16(reinterpret_cast<UA_LDS bf16x4*>(a_lo));
+  const bf16x4 y = __builtin_amdgcn_ds_read_tr16_b64_v4bf16(reinterpret_cast<UA_LDS bf16x4*>(a_hi));
+  return __builtin_shufflevector(x, y, 0, 1, 2, 3, 4, 5, 6, 7);
+}
+// buffer_load_dwordx4 ... lds with the LDS destination (wave-uniform) in M0; see dma16_buf.
+__device__ __forceinline__ void dma16_abs(u32x4 rsrc, uint32_t lds_addr, int voff, int soff) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
+               :: "s"(lds_addr), "v"(voff), "s"(rsrc), "s"(soff));
+}
+__device__ __forceinline__ u32x4 make_rsrc_words(const void* base, uint32_t bytes) {
+  const uint64_t a = reinterpret_cast<uint64_t>(base);
+  u32x4 r;
+  r[0] = __builtin_amdgcn_readfirstlane((uint32_t)a);
+  r[1] = __builtin_amdgcn_readfirstlane((uint32_t)(a >> 32) & 0xffffu);
+  r[2] = __builtin_amdgcn_readfirstlane(bytes);
+  r[3] = 0x00020000u;
+  return r;
+}
+
+// Per-lane absolute LDS addresses (stage 0, first 32-row block) of one wave group.
+struct DkdvAddr {
+  uint32_t nat[8];      // 128-bit row fragments of the operand that is read row-wise
+  uint32_t tr[4][2];    // transposing reads of the other operand
+  uint32_t p;           // this lane's 32 bytes of P per block
+  uint32_t stat;        // this lane half's 4 consecutive row statistics
+};
+
+// A block of 8 MFMAs reads 8 operand fragments from LDS.  Every block is split in two calls: the
+// first issues the reads of its first fragments (and, for a row-wise block, the 4 reads that
+// start the accumulator from the rows' statistic), the second runs the MFMAs, each preceded by
+// the read of the fragment kAhead positions later.  The first call of block n+1 is placed ahead
+// of the second call of block n, so a block never starts by waiting for LDS.
+constexpr int kTrAhead = 3, kNatAhead = 4;
+
+// Transposed operand: acc[mbd] += X^T * bfrag[t], 2 steps of 16 rows x 4 d-blocks.
+template <int kImm>
+__device__ __forceinline__ bf16x8 dkdv_tr_frag(const DkdvAddr& ad, int i) {
+  return lds_abs_tr_pair(ad.tr[i & 3][0] + (kImm + 16 * (i >> 2) * kRowBytes), ad.tr[i & 3][1] + (kImm + 16 * (i >> 2) * kRowBytes));
+}
+template <int kImm>
+__device__ __forceinline__ void dkdv_tr_first(const DkdvAddr& ad, bf16x8 (&fr)[8]) {
 #pragma unroll
-  for (int i = 0; i < kAhead; ++i)
-    fr[i] = read_tr_pair(sX + 16 * (i >> 2) * kRowBytes, lo.tr[i & 3][0] + blk, lo.tr[i & 3][1] + blk);
-  __builtin_amdgcn_sched_group_barrier(0x100, 2 * kAhead, 0);
+  for (int i = 0; i < kTrAhead; ++i) fr[i] = dkdv_tr_frag<kImm>(ad, i);
+  __builtin_amdgcn_sched_group_barrier(0x100, 2 * kTrAhead, 0);
+}
+template <int kImm>
+__device__ __forceinline__ void dkdv_tr_run(const DkdvAddr& ad, bf16x8 (&fr)[8], const bf16x8 (&bfrag)[2], f32x16 (&acc)[4]) {
 #pragma unroll
   for (int i = 0; i < 8; ++i) {
-    if (i + kAhead < 8) {
-      const int j = i + kAhead;
-      fr[j] = read_tr_pair(sX + 16 * (j >> 2) * kRowBytes, lo.tr[j & 3][0] + blk, lo.tr[j & 3][1] + blk);
-    }
+    if (i + kTrAhead < 8) fr[i + kTrAhead] = dkdv_tr_frag<kImm>(ad, i + kTrAhead);
     acc[i & 3] = mfma32(fr[i], bfrag[i >> 2], acc[i & 3]);
     __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-    __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+    if (i + kTrAhead < 8) __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
   }
 }
 
-// One 32x32 block: stat + X[rows 32*nb.., :] * frag^T over head_dim.  The accumulator starts
-// from the rows' statistic (4 x 128-bit LDS reads straight into it) instead of zero, which
-// folds the "- lse" / "- delta" of the pointwise step into the product.  The row fragments
-// are fetched kAhead reads ahead of the (dependent) MFMA chain.
-__device__ __forceinline__ f32x16 mfma_nat_block(const unsigned char* sX, const LaneOffsU& lo, int blk,
-                                                 const bf16x8 (&frag)[8], const float* stat_rows, int hi) {
-  constexpr int kAhead = 4;
-  bf16x8 fr[8];
+// Row-wise operand: one 32x32 block = stat + X[32 rows, :] * frag^T over head_dim.  The
+// accumulator starts from the rows' statistic instead of zero, which folds the "- lse" /
+// "- delta" of the pointwise step into the product.
+template <int kImm, int kStatImm>
+__device__ __forceinline__ void dkdv_nat_first(const DkdvAddr& ad, bf16x8 (&fr)[8], f32x16& acc) {
 #pragma unroll
-  for (int ks = 0; ks < kAhead; ++ks) fr[ks] = lds_read_b128(sX, lo.nat[ks] + blk);
-  f32x16 acc;
+  for (int ks = 0; ks < kNatAhead; ++ks) fr[ks] = lds_abs_b128(ad.nat[ks] + kImm);
   // element i: row 8*(i/4) + 4*hi + i%4 of the block
 #pragma unroll
   for (int g = 0; g < 4; ++g) {
-    const f32x4 v = *reinterpret_cast<const f32x4*>(stat_rows + 8 * g + 4 * hi);
+    const f32x4 v = *reinterpret_cast<const UA_LDS f32x4*>(ad.stat + (kStatImm + 32 * g));
     acc[4 * g] = v[0]; acc[4 * g + 1] = v[1]; acc[4 * g + 2] = v[2]; acc[4 * g + 3] = v[3];
   }
-  __builtin_amdgcn_sched_group_barrier(0x100, kAhead + 4, 0);
+  __builtin_amdgcn_sched_group_barrier(0x100, kNatAhead + 4, 0);
+}
+template <int kImm>
+__device__ __forceinline__ void dkdv_nat_run(const DkdvAddr& ad, bf16x8 (&fr)[8], const bf16x8 (&frag)[8], f32x16& acc) {
 #pragma unroll
   for (int ks = 0; ks < 8; ++ks) {
-    if (ks + kAhead < 8) fr[ks + kAhead] = lds_read_b128(sX, lo.nat[ks + kAhead] + blk);
+    if (ks + kNatAhead < 8) fr[ks + kNatAhead] = lds_abs_b128(ad.nat[ks + kNatAhead] + kImm);
     acc = mfma32(fr[ks], frag[ks], acc);
     __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-    __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+    if (ks + kNatAhead < 8) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
   }
-  return acc;
 }
 
 // P = exp2(scale_log2 * S') with S' = Q K^T - lse/scale (bf16, accumulator layout), written to
-// the hand-over slot.
-__device__ __forceinline__ void dkdv_p_from_s(f32x16 s, unsigned char* p_slot, float scale_log2,
+// the partner's slot.  nb = block of the query tile (0..3).
+template <int kPImm>
+__device__ __forceinline__ void dkdv_p_from_s(f32x16 s, const DkdvAddr& ad, float scale_log2,
                                               int nb, int hi, int key_l, bool causal, bf16x8 (&pb)[2]) {
   // element i: query row 32*nb + 8*(i/4) + 4*hi + i%4, key column key_l
   if (causal) {
@@ -149,64 +202,29 @@ __device__ __forceinline__ void dkdv_p_from_s(f32x16 s, unsigned char* p_slot, f
   }
 #pragma unroll
   for (int i = 0; i < 16; ++i) pb[i >> 3][i & 7] = (bf16)fast_exp2(s[i] * scale_log2);
-  *reinterpret_cast<bf16x8*>(p_slot) = pb[0];
-  *reinterpret_cast<bf16x8*>(p_slot + 1024) = pb[1];
+  *reinterpret_cast<UA_LDS bf16x8*>(ad.p + kPImm) = pb[0];
+  *reinterpret_cast<UA_LDS bf16x8*>(ad.p + (kPImm + 1024)) = pb[1];
 }
 
-// Group A, one query tile.  The MFMAs of S(nb+1) are issued before the vector unit turns S(nb)
-// into P(nb); then the barrier publishes P(nb) and dV takes it.
-__device__ __forceinline__ void dkdv_tile_a(const unsigned char* sQ, const unsigned char* sdO, const float* sLse,
-                                            unsigned char* sP, int& pslot, const bf16x8 (&kf)[8], f32x16 (&dv)[4],
-                                            const LaneOffsU& lo, float scale_log2, int lane, int hi, int wave,
-                                            int key_l, bool causal) {
-  unsigned char* mine = sP + wave * 2048 + lane * 16;
-  f32x16 s_cur = mfma_nat_block(sQ, lo, 0, kf, sLse, hi), s_next;
-  bf16x8 pb[2];
+// dS = P * dP' for one block, P (two 128-bit words per lane) read from the partner's slot.
+template <int kPImm>
+__device__ __forceinline__ void dkdv_p_read(const DkdvAddr& ad, u32x4 (&praw)[2]) {
+  praw[0] = *reinterpret_cast<const UA_LDS u32x4*>(ad.p + kPImm);
+  praw[1] = *reinterpret_cast<const UA_LDS u32x4*>(ad.p + (kPImm + 1024));
+}
+__device__ __forceinline__ void dkdv_ds_from_p(const u32x4 (&praw)[2], const f32x16& dp, bf16x8 (&dsb)[2]) {
 #pragma unroll
-  for (int nb = 0; nb < 4; ++nb) {     // 32 query rows at a time
-    if (nb < 3) s_next = mfma_nat_block(sQ, lo, (nb + 1) * 32 * kRowBytes, kf, sLse + 32 * (nb + 1), hi);
-    dkdv_p_from_s(s_cur, mine + pslot * kPBlockBytes, scale_log2, nb, hi, key_l, causal, pb);
-    pslot = pslot == 2 ? 0 : pslot + 1;
-    lds_barrier();                     // P of block nb is visible to the partner wave
-    mfma_tr_block(sdO, lo, nb * 32 * kRowBytes, pb, dv);
-    s_cur = s_next;
+  for (int i = 0; i < 16; ++i) {
+    const uint32_t w = praw[i >> 3][(i & 7) >> 1];
+    const float pv = __uint_as_float((i & 1) ? (w & 0xffff0000u) : (w << 16));
+    dsb[i >> 3][i & 7] = (bf16)(pv * dp[i]);
   }
 }
-
-// Group B, one query tile: dP'(nb+1) = dO V^T - delta is issued before dS(nb) = P(nb) * dP'(nb)
-// is formed.
-__device__ __forceinline__ void dkdv_tile_b(const unsigned char* sQ, const unsigned char* sdO, const float* sNegDelta,
-                                            const unsigned char* sP, int& pslot, const bf16x8 (&vf)[8], f32x16 (&dk)[4],
-                                            const LaneOffsU& lo, int lane, int hi, int wave) {
-  const unsigned char* mine = sP + wave * 2048 + lane * 16;
-  f32x16 dp_cur = mfma_nat_block(sdO, lo, 0, vf, sNegDelta, hi), dp_next;
-#pragma unroll
-  for (int nb = 0; nb < 4; ++nb) {
-    if (nb < 3) dp_next = mfma_nat_block(sdO, lo, (nb + 1) * 32 * kRowBytes, vf, sNegDelta + 32 * (nb + 1), hi);
-    lds_barrier();                     // the partner's P of this block has been written
-    const unsigned char* src = mine + pslot * kPBlockBytes;
-    pslot = pslot == 2 ? 0 : pslot + 1;
-    u32x4 praw[2];
-    praw[0] = *reinterpret_cast<const u32x4*>(src);
-    praw[1] = *reinterpret_cast<const u32x4*>(src + 1024);
-    bf16x8 dsb[2];
-#pragma unroll
-    for (int i = 0; i < 16; ++i) {
-      const uint32_t w = praw[i >> 3][(i & 7) >> 1];
-      const float pv = __uint_as_float((i & 1) ? (w & 0xffff0000u) : (w << 16));
-      dsb[i >> 3][i & 7] = (bf16)(pv * dp_cur[i]);
-    }
-    mfma_tr_block(sQ, lo, nb * 32 * kRowBytes, dsb, dk);
-    dp_cur = dp_next;
-  }
-}
-
-struct DkdvStage { unsigned char* q; unsigned char* dout; float* stat; };
 
 // The whole key-tile column for one wave group (kGroupB: dK, else dV).  Both groups execute the
 // same sequence of barriers.
 template <bool kGroupB>
-__device__ __forceinline__ void dkdv_run(const BwdParams& p, const DkdvStage (&stg)[2], unsigned char* sP, int kt, int b,
+__device__ __forceinline__ void dkdv_run(const BwdParams& p, uint32_t lds_base, int kt, int b,
                                          int h, int tid, int lane, int wave8) {
   const int wave = wave8 & 3, l32 = lane & 31, hi = lane >> 5;
   const int64_t seq_q = (int64_t)p.n_qtiles * kTile;
@@ -221,14 +239,34 @@ __device__ __forceinline__ void dkdv_run(const BwdParams& p, const DkdvStage (&s
   f32x16 acc[4];       // group A: dV^T, group B: dK^T
 #pragma unroll
   for (int i = 0; i < 4; ++i) acc[i] = f32x16{0};
+  f32x16 dp[2];        // group B: dP' of the half tile it finishes in the next step
+  dp[0] = f32x16{0};
+  dp[1] = f32x16{0};
 
   const bf16* qbase = p.q + b * p.qs.b + h * p.qs.h;
   const bf16* dobase = p.dout + b * p.ds.b + h * p.ds.h;
   const float* lse_row = p.lse + ((int64_t)b * p.n_heads + h) * seq_q;
   const float* delta_row = p.delta + ((int64_t)b * p.n_heads + h) * seq_q;
-  const TrLane tr(lane);
-  const LaneOffsU lo(l32, hi, tr);
   const int key_l = wave * 32 + l32;
+
+  // group A reads Q row-wise (S) and dO transposed (dV); group B reads dO row-wise (dP) and Q
+  // transposed (dK)
+  DkdvAddr ad;
+  {
+    const TrLane tr(lane);
+    const LaneOffsU lo(l32, hi, tr);
+    const uint32_t nat_ring = lds_base + (kGroupB ? kRingDO : kRingQ), tr_ring = lds_base + (kGroupB ? kRingQ : kRingDO);
+#pragma unroll
+    for (int ks = 0; ks < 8; ++ks) { ad.nat[ks] = nat_ring + lo.nat[ks]; keep_in_register(ad.nat[ks]); }
+#pragma unroll
+    for (int m = 0; m < 4; ++m)
+#pragma unroll
+      for (int t = 0; t < 2; ++t) { ad.tr[m][t] = tr_ring + lo.tr[m][t]; keep_in_register(ad.tr[m][t]); }
+    ad.p = lds_base + kRingP + wave * 2048 + lane * 16;
+    keep_in_register(ad.p);
+    ad.stat = lds_base + kRingStat + (kGroupB ? kHalf * 4 : 0) + 16 * hi;
+    keep_in_register(ad.stat);
+  }
 
   const int q_stride = (int)p.qs.s, do_stride = (int)p.ds.s;
   int qoff[2], dooff[2];
@@ -237,91 +275,135 @@ __device__ __forceinline__ void dkdv_run(const BwdParams& p, const DkdvStage (&s
   const int q_half = kHalf * q_stride * 2, do_half = kHalf * do_stride * 2;
   const uint32_t q_extent = (uint32_t)((kTile - 1) * q_stride + kHeadDim) * 2;
   const uint32_t do_extent = (uint32_t)((kTile - 1) * do_stride + kHeadDim) * 2;
-  auto qtile = [&](int e) { return min(max(sload(p.idx, e), 0), p.n_qtiles - 1); };
-  // rows' statistics, staged in the form the accumulators start from: threads 0..127 carry
+  const int e0 = sload(p.ptr, kt), e1 = sload(p.ptr, kt + 1);
+  const int n_half = 2 * (e1 - e0);
+  // half tile i = half (i & 1) of list entry e0 + i / 2.  The list entry (query tile, causal
+  // flag) of half tile i+1 is fetched one step before it is needed, so that no step starts by
+  // waiting for a scalar load.
+  auto entry = [&](int i) {           // query tile | causal flag << 30
+    const int e = min(e0 + (i >> 1), e1 - 1);
+    return min(max(sload(p.idx, e), 0), p.n_qtiles - 1) | (sload(p.flag, e) << 30);
+  };
+  // rows' statistics, staged in the form the accumulators start from: threads 0..63 carry
   // -lse/softmax_scale (lse = -inf, a row without keys, stays -inf so that P = 0), threads
-  // 128..255 carry -delta
+  // 64..127 carry -delta
+  // (the raw value is only touched when it is stored to LDS at the end of a step: no wait for
+  // the global load may land between the copies' issue and the step's work)
   const float neg_inv_scale = -1.f / p.scale;
-  auto load_stat = [&](int qt) {
+  const float* stat_src = (tid < kHalf ? lse_row : delta_row) + (tid & (kHalf - 1));
+  auto load_stat = [&](int i, int qt) {
     float x = 0.f;
-    if (tid < 2 * kTile) {
-      x = tid < kTile ? lse_row[qt * kTile + tid] : delta_row[qt * kTile + tid - kTile];
-      x = tid < kTile ? ((x == -INFINITY) ? -INFINITY : x * neg_inv_scale) : -x;
-    }
+    if (tid < 2 * kHalf) x = stat_src[qt * kTile + (i & 1) * kHalf];
     return x;
   };
-  auto stage = [&](int qt, const DkdvStage& st) {
-    const __amdgpu_buffer_rsrc_t rq = make_rsrc(qbase + (int64_t)qt * kTile * q_stride, q_extent);
-    const __amdgpu_buffer_rsrc_t rd = make_rsrc(dobase + (int64_t)qt * kTile * do_stride, do_extent);
-    dma_half_tile_buf<8>(st.q, rq, qoff, 0, wave8);
-    dma_half_tile_buf<8>(st.q + kHalfBytes, rq, qoff, q_half, wave8);
-    dma_half_tile_buf<8>(st.dout, rd, dooff, 0, wave8);
-    dma_half_tile_buf<8>(st.dout + kHalfBytes, rd, dooff, do_half, wave8);
+  const uint32_t dma_lds = __builtin_amdgcn_readfirstlane(lds_base + wave8 * 1024);
+  auto copy_in = [&](int i, int qt, int stage) {       // 8 waves x 2 copies x 1 KiB per operand
+    const u32x4 rq = make_rsrc_words(qbase + (int64_t)qt * kTile * q_stride, q_extent);
+    const u32x4 rd = make_rsrc_words(dobase + (int64_t)qt * kTile * do_stride, do_extent);
+    const int sq = __builtin_amdgcn_readfirstlane((i & 1) * q_half), sd = __builtin_amdgcn_readfirstlane((i & 1) * do_half);
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      dma16_abs(rq, dma_lds + kRingQ + stage * kHalfBytes + j * 8192, qoff[j], sq);
+      dma16_abs(rd, dma_lds + kRingDO + stage * kHalfBytes + j * 8192, dooff[j], sd);
+    }
   };
-  // Both groups advance the hand-over slot once per block: group A names the slot of the block
-  // it writes next (one ahead), group B the slot of the block it reads.
-  int pslot = 0;
-  auto tile = [&](const DkdvStage& st, bool causal) {
-    if (kGroupB) dkdv_tile_b(st.q, st.dout, st.stat + kTile, sP, pslot, frag, acc, lo, lane, hi, wave);
-    else         dkdv_tile_a(st.q, st.dout, st.stat, sP, pslot, frag, acc, lo, p.scale_log2, lane, hi, wave, key_l, causal);
+  auto put_stat = [&](int stage, float x) {
+    if (tid < 2 * kHalf) {
+      x = tid < kHalf ? ((x == -INFINITY) ? -INFINITY : x * neg_inv_scale) : -x;
+      *reinterpret_cast<UA_LDS float*>(lds_base + kRingStat + stage * kStatBytes + tid * 4) = x;
+    }
+  };
+  int ent[2] = {0, 0};
+  // One step on stage kCur = i mod 3: copies for half tile i+1 go in flight into the next stage;
+  // group A works on half tile i; group B finishes half tile i-1 (previous stage) and computes dP'
+  // of half tile i.
+  auto step = [&](int i, auto cur_tag) {
+    constexpr int kCur = decltype(cur_tag)::value, kPrev = (kCur + 2) % 3, kNext = (kCur + 1) % 3;
+    if (i > n_half) return;            // workgroup-uniform: the column is done
+    const bool more = i + 1 < n_half;
+    const int ent_cur = ent[0], ent_next = ent[1];     // entries of half tiles i and i+1
+    ent[0] = ent_next;
+    ent[1] = entry(i + 2);
+    float stat = 0.f;
+    if (more) {
+      stat = load_stat(i + 1, ent_next & 0x3fffffff);
+      copy_in(i + 1, ent_next & 0x3fffffff, kNext);
+    }
+    constexpr int kQ0 = kCur * kHalfBytes, kQ1 = kQ0 + 32 * kRowBytes;          // blocks of this half tile
+    constexpr int kPrev0 = kPrev * kHalfBytes, kPrev1 = kPrev0 + 32 * kRowBytes;  // blocks of the previous one
+    bf16x8 f0[8], f1[8];       // operand fragments of the block being run / the block after it
+    if (kGroupB) {
+      // unconditional: in step 0 P and dP' are zero (dK += 0), in the last step the new dP' is
+      // computed from stale rows and never used
+      u32x4 p0[2], p1[2];
+      bf16x8 ds0[2], ds1[2];
+      dkdv_p_read<kPrev * kPHalfBytes>(ad, p0);
+      dkdv_p_read<kPrev * kPHalfBytes + kPBlockBytes>(ad, p1);
+      __builtin_amdgcn_sched_group_barrier(0x100, 4, 0);
+      dkdv_tr_first<kPrev0>(ad, f0);
+      dkdv_ds_from_p(p0, dp[0], ds0);
+      dkdv_ds_from_p(p1, dp[1], ds1);
+      dkdv_tr_first<kPrev1>(ad, f1);
+      dkdv_tr_run<kPrev0>(ad, f0, ds0, acc);
+      dkdv_nat_first<kQ0, kCur * kStatBytes>(ad, f0, dp[0]);
+      dkdv_tr_run<kPrev1>(ad, f1, ds1, acc);
+      dkdv_nat_first<kQ1, kCur * kStatBytes + 128>(ad, f1, dp[1]);
+      dkdv_nat_run<kQ0>(ad, f0, frag, dp[0]);
+      dkdv_nat_run<kQ1>(ad, f1, frag, dp[1]);
+    } else if (i < n_half) {
+      const bool causal = (ent_cur >> 30) != 0;
+      bf16x8 pb0[2], pb1[2];
+      f32x16 s0, s1;
+      dkdv_nat_first<kQ0, kCur * kStatBytes>(ad, f0, s0);
+      dkdv_nat_first<kQ1, kCur * kStatBytes + 128>(ad, f1, s1);
+      dkdv_nat_run<kQ0>(ad, f0, frag, s0);
+      dkdv_tr_first<kQ0>(ad, f0);
+      dkdv_nat_run<kQ1>(ad, f1, frag, s1);
+      dkdv_tr_first<kQ1>(ad, f1);
+      dkdv_p_from_s<kCur * kPHalfBytes>(s0, ad, p.scale_log2, 2 * (i & 1), hi, key_l, causal, pb0);
+      dkdv_p_from_s<kCur * kPHalfBytes + kPBlockBytes>(s1, ad, p.scale_log2, 2 * (i & 1) + 1, hi, key_l, causal, pb1);
+      dkdv_tr_run<kQ0>(ad, f0, pb0, acc);
+      dkdv_tr_run<kQ1>(ad, f1, pb1, acc);
+    }
+    if (more) put_stat(kNext, stat);
+    wait_vmem_all();
+    __syncthreads();     // next stage has landed, P of half tile i is visible, everyone is done with the previous stage
   };
 
-  const int e0 = sload(p.ptr, kt), e1 = sload(p.ptr, kt + 1);
-  if (e0 < e1) {
-    const int qt = qtile(e0);
-    const float st0 = load_stat(qt);
-    if (tid < 2 * kTile) stg[0].stat[tid] = st0;
-    stage(qt, stg[0]);
+  if (n_half > 0) {
+    ent[0] = entry(0);
+    ent[1] = entry(1);
+    const float st0 = load_stat(0, ent[0] & 0x3fffffff);
+    copy_in(0, ent[0] & 0x3fffffff, 0);
+    put_stat(0, st0);
   }
-  // entries are taken two at a time, even ones through stage 0 and odd ones through stage 1,
-  // so that every LDS access names its stage statically (reads of one stage then need not
-  // wait for the copies in flight into the other)
-  for (int e = e0; e < e1; e += 2) {
-    const bool has1 = e + 1 < e1, has2 = e + 2 < e1;
-    float stat = 0.f;
-    wait_vmem_all();
-    __syncthreads();                       // stage 0 landed; everyone is done with stage 1
-    if (has1) {
-      const int qt = qtile(e + 1);
-      stat = load_stat(qt);
-      stage(qt, stg[1]);
-    }
-    tile(stg[0], sload(p.flag, e) != 0);
-    if (!has1) break;
-    if (tid < 2 * kTile) stg[1].stat[tid] = stat;
-    wait_vmem_all();
-    __syncthreads();                       // stage 1 landed; everyone is done with stage 0
-    if (has2) {
-      const int qt = qtile(e + 2);
-      stat = load_stat(qt);
-      stage(qt, stg[0]);
-    }
-    tile(stg[1], sload(p.flag, e + 1) != 0);
-    if (has2 && tid < 2 * kTile) stg[0].stat[tid] = stat;
+  // step 0 lets group B "finish" a half tile that does not exist: its P (stage 2) must be zero
+  for (int o = tid * 16; o < kPHalfBytes; o += 512 * 16)
+    *reinterpret_cast<UA_LDS u32x4*>(lds_base + kRingP + 2 * kPHalfBytes + o) = u32x4{0, 0, 0, 0};
+  wait_vmem_all();
+  __syncthreads();
+  // steps 0 .. n_half (the last one only lets group B finish), three at a time so that the
+  // stage is a compile-time constant
+  for (int i = 0; i <= n_half; i += 3) {
+    step(i, std::integral_constant<int, 0>{});
+    step(i + 1, std::integral_constant<int, 1>{});
+    step(i + 2, std::integral_constant<int, 2>{});
   }
   if (kGroupB) store_acc_t(p.out0 + b * p.o0s.b + (int64_t)krow * p.o0s.s + h * p.o0s.h, acc, p.scale, hi);
   else         store_acc_t(p.out1 + b * p.o1s.b + (int64_t)krow * p.o1s.s + h * p.o1s.h, acc, 1.f, hi);
 }
 
 __global__ __launch_bounds__(512) void dkdv_kernel(const BwdParams p) {
-  // two stages (Q tile, dO tile, the rows' lse and delta)
-  __shared__ __attribute__((aligned(1024))) unsigned char sQ0[kTileBytes];
-  __shared__ __attribute__((aligned(1024))) unsigned char sdO0[kTileBytes];
-  __shared__ __attribute__((aligned(1024))) unsigned char sQ1[kTileBytes];
-  __shared__ __attribute__((aligned(1024))) unsigned char sdO1[kTileBytes];
-  __shared__ __attribute__((aligned(1024))) unsigned char sP[3 * kPBlockBytes];
-  __shared__ __attribute__((aligned(16))) float sStat0[2 * kTile];
-  __shared__ __attribute__((aligned(16))) float sStat1[2 * kTile];
-
+  __shared__ __attribute__((aligned(1024))) unsigned char smem[kDkdvLdsBytes];
+  const uint32_t lds_base = (uint32_t)(uintptr_t)(UA_LDS unsigned char*)smem;
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave8 = __builtin_amdgcn_readfirstlane(tid >> 6);      // 0..7
   int pos, bh;
   map_block(blockIdx.x, p.batch * p.n_heads, p.heads_per_xcd, p.n_ktiles, pos, bh);
   const int kt = sload(p.order, pos);
   const int b = bh / p.n_heads, h = bh % p.n_heads;
-  const DkdvStage stg[2] = {{sQ0, sdO0, sStat0}, {sQ1, sdO1, sStat1}};
-  if (wave8 >= 4) dkdv_run<true>(p, stg, sP, kt, b, h, tid, lane, wave8);
-  else            dkdv_run<false>(p, stg, sP, kt, b, h, tid, lane, wave8);
+  if (wave8 >= 4) dkdv_run<true>(p, lds_base, kt, b, h, tid, lane, wave8);
+  else            dkdv_run<false>(p, lds_base, kt, b, h, tid, lane, wave8);
 }
 
 // dQ: one 64-key half tile for this wave's 32 query rows.
