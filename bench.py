@@ -27,7 +27,7 @@ FLOP_PER_CLK_PER_CU = 4096        # dense bf16 MFMA, CDNA4
 
 # HBM bytes per launch of the dominant kernel, from profiles/hbm_traffic_<workload>.txt
 # (rocprofv3 --pmc FETCH_SIZE x 2.0 + WRITE_SIZE x 1.0, scaling explained there).
-TRAFFIC_BYTES = {("c3", "dkdv_kernel"): 42.57e9, ("c5", "fwd_kernel"): 10.88e9}
+TRAFFIC_BYTES = {("c3", "dkdv_kernel"): 41.84e9, ("c5", "fwd_kernel"): 10.85e9}
 
 
 def log(*a):
