@@ -48,13 +48,6 @@ __device__ __forceinline__ void store_acc_t(bf16* row_ptr, const f32x16 (&acc)[4
 constexpr int kHalf = 64;
 constexpr int kHalfBytes = kHalf * kRowBytes;      // 16 KiB
 
-// Stage one full [128][128] bf16 tile (two half tiles) with asynchronous copies, 256 threads.
-__device__ __forceinline__ void dma_tile_buf(unsigned char* lds, __amdgpu_buffer_rsrc_t r, const int (&voff)[4],
-                                             int half_bytes, int wave) {
-  dma_half_tile_buf<4>(lds, r, voff, 0, wave);
-  dma_half_tile_buf<4>(lds + kHalfBytes, r, voff, half_bytes, wave);
-}
-
 // Per-lane LDS byte offsets into a tile held in the universal layout, for the first 32-row
 // block; later blocks add 32*kRowBytes per block (the XOR term repeats every 16 rows).
 struct LaneOffsU {
@@ -70,12 +63,6 @@ struct LaneOffsU {
     }
   }
 };
-__device__ __forceinline__ bf16x8 read_tr_pair(const unsigned char* smem, int off_lo, int off_hi) {
-  const bf16x4 a = lds_read_tr16_b64(smem, off_lo);
-  const bf16x4 b = lds_read_tr16_b64(smem, off_hi);
-  return __builtin_shufflevector(a, b, 0, 1, 2, 3, 4, 5, 6, 7);
-}
-
 // ---- dK/dV ------------------------------------------------------------------------------------
 // The workgroup has 8 wavefronts in two groups of 4; wave w of either group owns key rows
 // 32w..32w+31 of the key tile, and each SIMD hosts one wave of each group.  Work is handed out

@@ -85,9 +85,6 @@ __device__ __forceinline__ bf16x8 lds_read_tr_frag(const unsigned char* smem, co
 }
 
 __device__ __forceinline__ void wait_vmem_all() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
-// Workgroup barrier that orders LDS traffic only: unlike __syncthreads() it does not wait for
-// the asynchronous global->LDS copies still in flight (they target another stage).
-__device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
 // Keeps a wave-uniform branch a branch (the optimiser may not turn its body into selects).
 __device__ __forceinline__ void keep_branch() { asm volatile("" ::: "memory"); }
 
