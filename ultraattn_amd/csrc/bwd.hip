@@ -364,9 +364,12 @@ __device__ __forceinline__ void dkdv_run(const BwdParams& p, uint32_t lds_base, 
     copy_in(0, ent[0] & 0x3fffffff, 0);
     put_stat(0, st0);
   }
-  // step 0 lets group B "finish" a half tile that does not exist: its P (stage 2) must be zero
+  // step 0 lets group B "finish" a half tile that does not exist: its P and its Q rows (stage 2)
+  // must be zero, not whatever the LDS held (0 x NaN would reach dK)
   for (int o = tid * 16; o < kPHalfBytes; o += 512 * 16)
     *reinterpret_cast<UA_LDS u32x4*>(lds_base + kRingP + 2 * kPHalfBytes + o) = u32x4{0, 0, 0, 0};
+  for (int o = tid * 16; o < kHalfBytes; o += 512 * 16)
+    *reinterpret_cast<UA_LDS u32x4*>(lds_base + kRingQ + 2 * kHalfBytes + o) = u32x4{0, 0, 0, 0};
   wait_vmem_all();
   __syncthreads();
   // steps 0 .. n_half (the last one only lets group B finish), three at a time so that the
