@@ -142,3 +142,24 @@ def test_full_size_sampled_rows(cfg):
                                 v[:, key:key + 1, h:h + 1], lse[:, h:h + 1, vis], delta[:, h:h + 1, vis], SCALE)
         assert (dk[0, key, h].float() - rk[0, 0, 0]).abs().max().item() <= ATOL_O, (key, h)
         assert (dv[0, key, h].float() - rv[0, 0, 0]).abs().max().item() <= ATOL_O, (key, h)
+
+
+def test_stale_lds_contents_do_not_leak_into_gradients():
+    """The kernels stage operands in LDS rings and may touch a stage before its first fill; what an
+    earlier launch left there (here: NaN everywhere, from a backward over NaN inputs that fills
+    every CU) must not reach any result."""
+    big = np.ones((8, 8), np.uint8)
+    nan = torch.full((1, 8 * 128, 64, 128), float("nan"), dtype=torch.bfloat16, device=DEV)
+    lse_nan = torch.zeros(1, 64, 8 * 128, dtype=torch.float32, device=DEV)
+    for _ in range(2):
+        ops.bsa_fwd(nan, nan, nan, big, SCALE, block=128)
+        ops.bsa_bwd(nan, nan, nan, nan, None, lse_nan, big, SCALE, block=128, softmax_d=lse_nan)
+    torch.cuda.synchronize()
+    for mask in (np.array([[1, 0], [0, 0]], np.uint8), np.array([[2, 0, 0], [1, 2, 0], [1, 0, 1]], np.uint8),
+                 np.zeros((2, 2), np.uint8)):
+        q, k, v, do = seeded_inputs(mask, 128, 7, nh=8)
+        o, lse, dq, dk, dv = run_fwd_bwd(q, k, v, do, mask, 128)
+        ro, rl, rq, rk, rv = oracle_fwd_bwd(q, k, v, do, mask, 128)
+        for got, ref in ((o, ro), (dq, rq), (dk, rk), (dv, rv)):
+            assert torch.isfinite(got.float()).all()
+            assert max_abs(got, ref) <= ATOL_O

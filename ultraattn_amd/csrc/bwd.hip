@@ -268,6 +268,7 @@ __device__ __forceinline__ void dkdv_run(const BwdParams& p, uint32_t lds_base, 
   // flag) of half tile i+1 is fetched one step before it is needed, so that no step starts by
   // waiting for a scalar load.
   auto entry = [&](int i) {           // query tile | causal flag << 30
+    if (n_half == 0) return 0;        // an empty column owns no list entry (the arrays may be NULL)
     const int e = min(e0 + (i >> 1), e1 - 1);
     return min(max(sload(p.idx, e), 0), p.n_qtiles - 1) | (sload(p.flag, e) << 30);
   };
