@@ -391,7 +391,7 @@ __global__ __launch_bounds__(512) void dkdv_kernel(const BwdParams p) {
   const int wave8 = __builtin_amdgcn_readfirstlane(tid >> 6);      // 0..7
   int pos, bh;
   map_block(blockIdx.x, p.batch * p.n_heads, p.heads_per_xcd, p.n_ktiles, pos, bh);
-  const int kt = sload(p.order, pos);
+  const int kt = min(max(sload(p.order, pos), 0), p.n_ktiles - 1);
   const int b = bh / p.n_heads, h = bh % p.n_heads;
   if (wave8 >= 4) dkdv_run<true>(p, lds_base, kt, b, h, tid, lane, wave8);
   else            dkdv_run<false>(p, lds_base, kt, b, h, tid, lane, wave8);
@@ -467,7 +467,7 @@ __global__ __launch_bounds__(256, 2) void dq_kernel(const BwdParams p) {
   const int l32 = lane & 31, hi = lane >> 5;
   int pos, bh;
   map_block(blockIdx.x, p.batch * p.n_heads, p.heads_per_xcd, p.n_qtiles, pos, bh);
-  const int qt = sload(p.order, pos);
+  const int qt = min(max(sload(p.order, pos), 0), p.n_qtiles - 1);
   const int b = bh / p.n_heads, h = bh % p.n_heads;
   const int64_t seq_q = (int64_t)p.n_qtiles * kTile;
 

@@ -143,7 +143,7 @@ __global__ __launch_bounds__(256, 2) void fwd_kernel(const FwdParams p) {
   const int l32 = lane & 31, hi = lane >> 5;
   int pos, bh;
   map_block(blockIdx.x, p.batch * p.n_heads, p.heads_per_xcd, p.n_qtiles, pos, bh);
-  const int qt = sload(p.q_order, pos);
+  const int qt = min(max(sload(p.q_order, pos), 0), p.n_qtiles - 1);
   const int b = bh / p.n_heads, h = bh % p.n_heads;
 
   const bf16* kbase = p.k + b * p.ks.b + h * p.ks.h;
