@@ -34,6 +34,26 @@ def log(*a):
     print(*a, file=sys.stderr, flush=True)
 
 
+_probe_lib = None
+
+
+def probe_lib():
+    """libbench_probe.so: the benchmark's own device probes (not part of the product library)."""
+    global _probe_lib
+    if _probe_lib is None:
+        import ctypes
+        path = os.path.join(ROOT, "libbench_probe.so")
+        if not os.path.exists(path):
+            sys.exit(f"{path} is missing: build it with `python -m ultraattn_amd.build`")
+        lib = ctypes.CDLL(path)
+        vp, ci = ctypes.c_void_p, ctypes.c_int
+        lib.bench_probe_mfma.restype, lib.bench_probe_mfma.argtypes = ci, [vp, vp, ci, ci, vp]
+        lib.bench_stream_mix.restype = ci
+        lib.bench_stream_mix.argtypes = [ctypes.POINTER(vp), ci, vp, ctypes.c_int64, ci, ci, vp]
+        _probe_lib = lib
+    return _probe_lib
+
+
 def workload_mask(name):
     from ultraattn_amd import masks
     return {"c2": masks.config_causal(64), "c3": masks.config_strided(), "c4": masks.config_global_local(),
@@ -146,14 +166,14 @@ def time_bwd_kernels(name, steps):
         _lib.check(lib.ua_bsa_bwd_dkdv(q.data_ptr(), k.data_ptr(), v.data_ptr(), do.data_ptr(), lse.data_ptr(),
                                        delta.data_ptr(), dk.data_ptr(), dv.data_ptr(), d["col_ptr"].data_ptr(),
                                        d["row_idx"].data_ptr(), d["cflag"].data_ptr(), d["k_order"].data_ptr(),
-                                       1, HEADS, tl.n_qtiles, tl.n_ktiles, 128, s3(q), s3(k), s3(v), s3(do), s3(dk),
+                                       1, HEADS, tl.n_qtiles, tl.n_ktiles, tl.nnz, 128, s3(q), s3(k), s3(v), s3(do), s3(dk),
                                        s3(dv), SCALE, st), "dkdv")
 
     def dqk():
         _lib.check(lib.ua_bsa_bwd_dq(q.data_ptr(), k.data_ptr(), v.data_ptr(), do.data_ptr(), lse.data_ptr(),
                                      delta.data_ptr(), dq.data_ptr(), d["row_ptr"].data_ptr(), d["col_idx"].data_ptr(),
                                      d["flag"].data_ptr(), d["q_order"].data_ptr(), 1, HEADS, tl.n_qtiles,
-                                     tl.n_ktiles, 128, s3(q), s3(k), s3(v), s3(do), s3(dq), SCALE, st), "dq")
+                                     tl.n_ktiles, tl.nnz, 128, s3(q), s3(k), s3(v), s3(do), s3(dq), SCALE, st), "dq")
     dkdv(); dqk()
     torch.cuda.synchronize()
     t = Timer(torch, ["dkdv", "dq"])
@@ -343,8 +363,8 @@ def run_power(name):
     runs = {
         "forward": lambda: ops.bsa_fwd(q, k, v, tl, SCALE, out=o, lse=lse),
         "backward": lambda: ops.bsa_bwd(do, q, k, v, None, lse, tl, SCALE, dq=dq, dk=dk, dv=dv, softmax_d=delta),
-        "mfma_random_operands": lambda: lib.ua_probe_mfma(rnd.data_ptr(), sink.data_ptr(), 512, 20000, st),
-        "mfma_constant_operands": lambda: lib.ua_probe_mfma(one.data_ptr(), sink.data_ptr(), 512, 20000, st),
+        "mfma_random_operands": lambda: probe_lib().bench_probe_mfma(rnd.data_ptr(), sink.data_ptr(), 512, 20000, st),
+        "mfma_constant_operands": lambda: probe_lib().bench_probe_mfma(one.data_ptr(), sink.data_ptr(), 512, 20000, st),
         "copy_1GiB": lambda: dst.copy_(src),
     }
     out = {"workload": name}
@@ -356,8 +376,7 @@ def run_power(name):
 def probe_mfma(peak):
     """Sustained register-only MFMA rate with constant and with random operand bits."""
     import torch
-    from ultraattn_amd import _lib
-    lib = _lib.load()
+    lib = probe_lib()
     dev = "cuda:0"
     n_blocks, iters = 512, 40000
     out = torch.empty(n_blocks * 256, dtype=torch.float32, device=dev)
@@ -367,11 +386,11 @@ def probe_mfma(peak):
     res = {}
     st = torch.cuda.current_stream().cuda_stream
     for name, t in ops_.items():
-        _lib.check(lib.ua_probe_mfma(t.data_ptr(), out.data_ptr(), n_blocks, 2000, st), "ua_probe_mfma")
+        assert lib.bench_probe_mfma(t.data_ptr(), out.data_ptr(), n_blocks, 2000, st) == 0
         torch.cuda.synchronize()
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         e0.record()
-        _lib.check(lib.ua_probe_mfma(t.data_ptr(), out.data_ptr(), n_blocks, iters, st), "ua_probe_mfma")
+        assert lib.bench_probe_mfma(t.data_ptr(), out.data_ptr(), n_blocks, iters, st) == 0
         e1.record()
         torch.cuda.synchronize()
         ms = e0.elapsed_time(e1)

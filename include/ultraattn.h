@@ -21,6 +21,8 @@
  *    orchestrated_attn/orchestrated_attn_impl.py:91).  `*_order` is a permutation of the tile
  *    rows (columns) giving the launch order: rows much longer than average first, the rest in
  *    lexicographic order of their index lists so that rows sharing K/V tiles run together.
+ *    `nnz` is the number of entries of col_idx/flag (row_idx/cflag): the kernels clamp every
+ *    list bound to it, and only an empty list (nnz = 0) may pass NULL for those arrays.
  *  - Every function returns 0 (UA_OK) or a negative UA_ERR_* code; ua_strerror() names it.
  *    No exceptions cross this boundary and nothing aborts.
  *  - Functions hold no mutable global state and may be called from several host threads on
@@ -71,7 +73,10 @@ int ua_tilelist_build(const uint8_t *block_mask, int n_qblocks, int n_kblocks, i
 
 /* Device-side variant: `block_mask` and all outputs are DEVICE arrays (sizes as above, from
  * ua_tilelist_size on a host copy or an upper bound nnz <= n_qtiles*n_ktiles); `work` is a
- * device scratch of (n_qtiles + n_ktiles + 2) int32.  Produces the same arrays bit for bit. */
+ * device scratch of (n_qtiles + n_ktiles + 3) int32.  Produces the same arrays bit for bit.
+ * The mask cannot be validated without a synchronisation: an entry that is not 0, 1 or 2 is
+ * treated as EMPTY, and work[n_qtiles + n_ktiles + 2] receives the number of such entries (0 for
+ * a valid mask; the host builder returns UA_ERR_MASK instead) for the caller to read later.  */
 int ua_tilelist_build_device(const uint8_t *block_mask, int n_qblocks, int n_kblocks, int rate,
                              int32_t *row_ptr, int32_t *col_idx, uint8_t *flag,
                              int32_t *col_ptr, int32_t *row_idx, uint8_t *cflag,
@@ -86,7 +91,7 @@ int ua_tilelist_build_device(const uint8_t *block_mask, int n_qblocks, int n_kbl
 int ua_bsa_fwd(const void *q, const void *k, const void *v, void *o, float *lse,
                const int32_t *row_ptr, const int32_t *col_idx, const uint8_t *flag,
                const int32_t *q_order,
-               int batch, int n_heads, int n_qtiles, int n_ktiles, int head_dim,
+               int batch, int n_heads, int n_qtiles, int n_ktiles, int nnz, int head_dim,
                const int64_t *q_strides, const int64_t *k_strides, const int64_t *v_strides,
                const int64_t *o_strides, float softmax_scale, void *stream);
 
@@ -106,7 +111,7 @@ int ua_bsa_bwd_dkdv(const void *q, const void *k, const void *v, const void *dou
                     const float *lse, const float *delta, void *dk, void *dv,
                     const int32_t *col_ptr, const int32_t *row_idx, const uint8_t *cflag,
                     const int32_t *k_order,
-                    int batch, int n_heads, int n_qtiles, int n_ktiles, int head_dim,
+                    int batch, int n_heads, int n_qtiles, int n_ktiles, int nnz, int head_dim,
                     const int64_t *q_strides, const int64_t *k_strides, const int64_t *v_strides,
                     const int64_t *do_strides, const int64_t *dk_strides, const int64_t *dv_strides,
                     float softmax_scale, void *stream);
@@ -114,7 +119,7 @@ int ua_bsa_bwd_dq(const void *q, const void *k, const void *v, const void *dout,
                   const float *lse, const float *delta, void *dq,
                   const int32_t *row_ptr, const int32_t *col_idx, const uint8_t *flag,
                   const int32_t *q_order,
-                  int batch, int n_heads, int n_qtiles, int n_ktiles, int head_dim,
+                  int batch, int n_heads, int n_qtiles, int n_ktiles, int nnz, int head_dim,
                   const int64_t *q_strides, const int64_t *k_strides, const int64_t *v_strides,
                   const int64_t *do_strides, const int64_t *dq_strides,
                   float softmax_scale, void *stream);
@@ -144,14 +149,6 @@ int ua_merge(const void *const *o_parts, const float *const *lse_parts, int n_pa
  * aligned, and must not overlap; 2*n_chunks*batch <= 65535.                                      */
 int ua_cols_gather(const void *src, void *dst, int n_chunks, int batch, int64_t inner_elems, void *stream);
 int ua_cols_scatter(const void *src, void *dst, int n_chunks, int batch, int64_t inner_elems, void *stream);
-
-/* ---- diagnostic (no counterpart in the reference) ----------------------------------------------
- * Runs n_blocks workgroups of 256 threads, each wave issuing 4 * iters register-only
- * v_mfma_f32_32x32x16_bf16 (32768 flop each) on the 512 x 16 bytes of operand bits at `operands`
- * (device, 16-byte aligned); `out` receives n_blocks * 256 floats.  Timed by the caller, it gives
- * the matrix pipe's sustained rate for those operand bits: the benchmark reports it beside the
- * attention kernels because the part's clock follows the power its operands make it draw.     */
-int ua_probe_mfma(const void *operands, float *out, int n_blocks, int iters, void *stream);
 
 #ifdef __cplusplus
 }

@@ -23,7 +23,8 @@ def test_header_symbols_are_exported(lib):
     names = declared_symbols()
     assert {"ua_bsa_fwd", "ua_bsa_bwd_dkdv", "ua_bsa_bwd_dq", "ua_bsa_bwd_delta", "ua_merge",
             "ua_tilelist_build", "ua_tilelist_size", "ua_tilelist_build_device", "ua_strerror",
-            "ua_version", "ua_probe_mfma"} <= set(names)
+            "ua_version"} <= set(names)
+    assert "ua_probe_mfma" not in names, "bench-only diagnostics stay out of the product ABI"
     raw = ctypes.CDLL(LIB_PATH)
     for n in names:
         assert hasattr(raw, n), f"{n} declared in include/ultraattn.h but not exported"
@@ -35,17 +36,21 @@ def test_argument_checks_without_gpu(lib):
     s = (ctypes.c_int64 * 3)(128 * 128, 128, 128)
     buf = np.zeros(64, np.uint8).ctypes.data // 16 * 16 + 16     # any aligned non-null address; never dereferenced
     # NULL q
-    assert lib.ua_bsa_fwd(None, buf, buf, buf, buf, buf, buf, buf, buf, 1, 1, 1, 1, 128, s, s, s, s, 0.1, None) == -1
+    assert lib.ua_bsa_fwd(None, buf, buf, buf, buf, buf, buf, buf, buf, 1, 1, 1, 1, 1, 128, s, s, s, s, 0.1, None) == -1
     # head_dim != 128
-    assert lib.ua_bsa_fwd(buf, buf, buf, buf, buf, buf, buf, buf, buf, 1, 1, 1, 1, 64, s, s, s, s, 0.1, None) == -3
+    assert lib.ua_bsa_fwd(buf, buf, buf, buf, buf, buf, buf, buf, buf, 1, 1, 1, 1, 1, 64, s, s, s, s, 0.1, None) == -3
     # non-positive scale
-    assert lib.ua_bsa_fwd(buf, buf, buf, buf, buf, buf, buf, buf, buf, 1, 1, 1, 1, 128, s, s, s, s, 0.0, None) == -3
+    assert lib.ua_bsa_fwd(buf, buf, buf, buf, buf, buf, buf, buf, buf, 1, 1, 1, 1, 1, 128, s, s, s, s, 0.0, None) == -3
     # sizes
-    assert lib.ua_bsa_fwd(buf, buf, buf, buf, buf, buf, buf, buf, buf, 0, 1, 1, 1, 128, s, s, s, s, 0.1, None) == -2
+    assert lib.ua_bsa_fwd(buf, buf, buf, buf, buf, buf, buf, buf, buf, 0, 1, 1, 1, 1, 128, s, s, s, s, 0.1, None) == -2
+    # a non-empty list needs col_idx and flag; a negative nnz is a shape error
+    assert lib.ua_bsa_fwd(buf, buf, buf, buf, buf, buf, None, buf, buf, 1, 1, 1, 1, 1, 128, s, s, s, s, 0.1, None) == -1
+    assert lib.ua_bsa_fwd(buf, buf, buf, buf, buf, buf, buf, None, buf, 1, 1, 1, 1, 1, 128, s, s, s, s, 0.1, None) == -1
+    assert lib.ua_bsa_fwd(buf, buf, buf, buf, buf, buf, buf, buf, buf, 1, 1, 1, 1, -1, 128, s, s, s, s, 0.1, None) == -2
     # misaligned pointer / stride not a multiple of 8
-    assert lib.ua_bsa_fwd(buf + 2, buf, buf, buf, buf, buf, buf, buf, buf, 1, 1, 1, 1, 128, s, s, s, s, 0.1, None) == -4
+    assert lib.ua_bsa_fwd(buf + 2, buf, buf, buf, buf, buf, buf, buf, buf, 1, 1, 1, 1, 1, 128, s, s, s, s, 0.1, None) == -4
     bad = (ctypes.c_int64 * 3)(128 * 128, 132, 128)
-    assert lib.ua_bsa_fwd(buf, buf, buf, buf, buf, buf, buf, buf, buf, 1, 1, 1, 1, 128, bad, s, s, s, 0.1, None) == -4
+    assert lib.ua_bsa_fwd(buf, buf, buf, buf, buf, buf, buf, buf, buf, 1, 1, 1, 1, 1, 128, bad, s, s, s, 0.1, None) == -4
     # merge: too many partials, bad seqlen
     arr = (ctypes.c_void_p * 17)(*([buf] * 17))
     assert lib.ua_merge(arr, arr, 17, buf, buf, 1, 16, 1, 128, None) == -3
@@ -55,8 +60,13 @@ def test_argument_checks_without_gpu(lib):
     # backward
     assert lib.ua_bsa_bwd_delta(buf, None, buf, 1, 16, 1, 128, s, s, None) == -1
     assert lib.ua_bsa_bwd_delta(buf, buf, buf, 1, 16, 1, 96, s, s, None) == -3
-    assert lib.ua_bsa_bwd_dq(buf, buf, buf, buf, buf, buf, None, buf, buf, buf, buf, 1, 1, 1, 1, 128,
+    assert lib.ua_bsa_bwd_dq(buf, buf, buf, buf, buf, buf, None, buf, buf, buf, buf, 1, 1, 1, 1, 1, 128,
                              s, s, s, s, s, 0.1, None) in (-1, -7)
+    # backward kernels: NULL index arrays with a non-empty list
+    assert lib.ua_bsa_bwd_dq(buf, buf, buf, buf, buf, buf, buf, buf, None, buf, buf, 1, 1, 1, 1, 1, 128,
+                             s, s, s, s, s, 0.1, None) == -1
+    assert lib.ua_bsa_bwd_dkdv(buf, buf, buf, buf, buf, buf, buf, buf, buf, buf, None, buf, 1, 1, 1, 1, 1, 128,
+                               s, s, s, s, s, s, 0.1, None) == -1
     for code in range(-7, 1):
         assert lib.ua_strerror(code) != b"unknown error code"
     assert lib.ua_strerror(-99) == b"unknown error code"

@@ -34,12 +34,14 @@ def test_device_builder_bit_exact(make, block):
 
 
 @pytest.mark.parametrize("causal", [False, True])
-@pytest.mark.parametrize("sq,sk", [(256, 256), (128, 384), (384, 384)])
+@pytest.mark.parametrize("sq,sk", [(256, 256), (128, 384), (384, 384), (384, 128)])
 def test_flash_attn_shim(causal, sq, sk):
     """Same call as fwd_comp_func / bwd_comp_func make (orchestrated_attn_impl.py:326-337,
-    578-596), checked against the oracle's dense tile."""
-    if causal and sq != sk:
-        pytest.skip("the reference only runs causal tiles on square diagonal chunks")
+    578-596), checked against the oracle's dense tile.  The reference only runs causal tiles
+    on square diagonal chunks; for Sq != Skv the shim follows flash-attn 2.1+'s bottom-right
+    alignment (query i sees key j iff j <= i + Skv - Sq), checked here against the oracle's
+    dense formula under that explicit element mask (rows without a visible key: O = 0,
+    LSE = -inf)."""
     g = torch.Generator().manual_seed(sq + sk)
     mk = lambda n: torch.randn(1, n, 3, 128, generator=g).to(torch.bfloat16)
     q, k, v, do = mk(sq), mk(sk), mk(sk), mk(sq)
@@ -49,16 +51,28 @@ def test_flash_attn_shim(causal, sq, sk):
                               return_softmax=False, out=out_buf)
     assert len(res) == 8 and res[0].data_ptr() == out_buf.data_ptr()
     O, lse = res[0], res[5]
-    ro, rl = ao.tile_fwd(q, k, v, SCALE, causal)
+    keep = torch.ones(sq, sk, dtype=torch.bool)
+    if causal:
+        keep = torch.arange(sk)[None, :] <= torch.arange(sq)[:, None] + (sk - sq)
+    ro, rl = ao.dense_fwd(q, k, v, SCALE, keep)
+    if sq == sk or not causal:
+        to_, tl_ = ao.tile_fwd(q, k, v, SCALE, causal)          # the square case is the reference's own
+        assert torch.equal(to_, ro) and torch.equal(tl_, rl)
     assert lse.shape == (1, 3, sq)
     assert max_abs(O, ro) <= ATOL_O and lse_rel_err(lse, rl) <= RTOL_LSE
     delta = ao.softmax_delta(ro, do).to(DEV)
+    # dq/dk/dv given: written in place and returned
     dq, dk, dv = torch.empty_like(qd), torch.empty_like(kd), torch.empty_like(vd)
-    _flash_attn_backward(dod, qd, kd, vd, qd, lse, dq, dk, dv, 0.0, SCALE, causal, (-1, -1), None, False,
-                         rng_state=None, softmax_d=delta)
+    ret = _flash_attn_backward(dod, qd, kd, vd, qd, lse, dq, dk, dv, 0.0, SCALE, causal, (-1, -1), None, False,
+                               rng_state=None, softmax_d=delta)
+    assert ret[0].data_ptr() == dq.data_ptr() and ret[1].data_ptr() == dk.data_ptr() and ret[2].data_ptr() == dv.data_ptr()
+    # dq/dk/dv = None (allowed by flash-attn's API): allocated by the shim and returned
+    ret2 = _flash_attn_backward(dod, qd, kd, vd, qd, lse, None, None, None, 0.0, SCALE, causal, (-1, -1), None, False,
+                                rng_state=None, softmax_d=delta)
     torch.cuda.synchronize()
-    rq, rk, rv = ao.tile_bwd(do, q, k, v, rl, ao.softmax_delta(ro, do), SCALE, causal)
-    assert max_abs(dq, rq) <= ATOL_O and max_abs(dk, rk) <= ATOL_O and max_abs(dv, rv) <= ATOL_O
+    rq, rk, rv = ao.dense_bwd_autograd(q, k, v, do, SCALE, keep)
+    for got in ((dq, dk, dv), ret2[:3]):
+        assert max_abs(got[0], rq) <= ATOL_O and max_abs(got[1], rk) <= ATOL_O and max_abs(got[2], rv) <= ATOL_O
 
 
 def test_shim_rejects_unsupported_features():

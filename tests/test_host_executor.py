@@ -1,6 +1,7 @@
 """Host logic of the executor and of the packed buffers (no GPU): kernel-key -> mask rules and
 the buffer layouts of the reference, checked by pointer arithmetic."""
 import json
+import math
 import os
 
 import numpy as np
@@ -72,3 +73,23 @@ def test_packed_layouts_match_the_reference_offsets():
     # a fused rectangle of n chunks is the first n*Sp tokens of the same buffer (benchmark.py:271-276)
     two = packed.InputRowFwd(buf, (B, 2 * S // 2, Nh, D))
     assert two.Q.data_ptr() == base
+
+
+def test_gradient_packs_accumulate_in_fp32():
+    """Eight partial gradients reduced one by one equal the fp32 sum rounded once
+    (ring_flash_attn/ring_flash_attn.py:110-118 accumulates partial dq/dk/dv in fp32); a bf16
+    running sum does not."""
+    shape = (1, 128, 2, 128)
+    g = torch.Generator().manual_seed(5)
+    parts = [torch.randn(2 * 128 * 2 * 128, generator=g).to(torch.bfloat16) for _ in range(8)]
+    want = torch.stack([p.float() for p in parts]).sum(0)
+    for cls in (packed.OutputRowBwd, packed.OutputColBwd):
+        n = math.prod(shape) * (2 if cls is packed.OutputColBwd else 1)
+        packs = [cls(p.clone(), shape) for p in parts]
+        for other in packs[1:]:
+            packs[0].reduce(other)
+        assert torch.equal(packs[0].data, want[:n].to(torch.bfloat16))
+        naive = parts[0][:n].clone()
+        for p in parts[1:]:
+            naive.add_(p[:n])
+        assert not torch.equal(naive, packs[0].data)

@@ -9,7 +9,11 @@ PKG_DIR = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(PKG_DIR, "csrc")
 LIB_NAME = "libultraattn_hip.so"
 LIB_PATH = os.path.join(PKG_DIR, LIB_NAME)
-SOURCES = ["api.hip", "tilelist.hip", "merge.hip", "glue.hip", "fwd.hip", "bwd.hip", "probe.hip"]
+SOURCES = ["api.hip", "tilelist.hip", "merge.hip", "glue.hip", "fwd.hip", "bwd.hip"]
+# benchmark-only probes (register-only MFMA loop, streaming-mix ceiling): built beside bench.py,
+# never linked into the product library
+BENCH_SRC = os.path.join(os.path.dirname(PKG_DIR), "bench_probe.hip")
+BENCH_LIB_PATH = os.path.join(os.path.dirname(PKG_DIR), "libbench_probe.so")
 # -packed-fp32-ops: keep the compiler from forming v_pk_{add,mul,fma}_f32 out of scalar code.
 HIPCC_FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-Wall", "-Wno-unused-result",
                "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
@@ -54,5 +58,18 @@ def build_library(verbose: bool = False, jobs: int = 4) -> str:
     return LIB_PATH
 
 
+def build_bench_probe(verbose: bool = False) -> str:
+    """Compile bench_probe.hip into libbench_probe.so at the repository root (used by bench.py only)."""
+    cmd = [hipcc_path(), *HIPCC_FLAGS, "-shared", BENCH_SRC, "-o", BENCH_LIB_PATH]
+    if verbose:
+        print(" ".join(cmd), flush=True)
+    r = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    if r.returncode != 0:
+        raise RuntimeError(f"hipcc failed on bench_probe.hip:\n{r.stdout}")
+    return BENCH_LIB_PATH
+
+
 if __name__ == "__main__":
     print(build_library(verbose="-v" in sys.argv))
+    if os.path.exists(BENCH_SRC):
+        print(build_bench_probe(verbose="-v" in sys.argv))

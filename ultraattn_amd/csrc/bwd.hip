@@ -26,7 +26,7 @@ struct BwdParams {
   const float* lse; const float* delta;
   bf16* out0; bf16* out1;                  // dkdv: dk, dv; dq: dq, unused
   const int32_t* ptr; const int32_t* idx; const uint8_t* flag; const int32_t* order;
-  int batch, n_heads, n_qtiles, n_ktiles;
+  int batch, n_heads, n_qtiles, n_ktiles, nnz;
   Strides3 qs, ks, vs, ds, o0s, o1s;
   float scale_log2, scale;
   int heads_per_xcd;
@@ -98,9 +98,11 @@ __device__ __forceinline__ bf16x8 lds_abs_tr_pair(uint32_t a_lo, uint32_t a_hi) 
   return __builtin_shufflevector(x, y, 0, 1, 2, 3, 4, 5, 6, 7);
 }
 // buffer_load_dwordx4 ... lds with the LDS destination (wave-uniform) in M0; see dma16_buf.
+// M0 is declared clobbered; "memory" is left out on purpose so that LDS reads of the other
+// stages may be scheduled across the copy (completion is awaited explicitly at the step's end).
 __device__ __forceinline__ void dma16_abs(u32x4 rsrc, uint32_t lds_addr, int voff, int soff) {
   asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
-               :: "s"(lds_addr), "v"(voff), "s"(rsrc), "s"(soff));
+               :: "s"(lds_addr), "v"(voff), "s"(rsrc), "s"(soff) : "m0");
 }
 __device__ __forceinline__ u32x4 make_rsrc_words(const void* base, uint32_t bytes) {
   const uint64_t a = reinterpret_cast<uint64_t>(base);
@@ -262,7 +264,7 @@ __device__ __forceinline__ void dkdv_run(const BwdParams& p, uint32_t lds_base, 
   const int q_half = kHalf * q_stride * 2, do_half = kHalf * do_stride * 2;
   const uint32_t q_extent = (uint32_t)((kTile - 1) * q_stride + kHeadDim) * 2;
   const uint32_t do_extent = (uint32_t)((kTile - 1) * do_stride + kHeadDim) * 2;
-  const int e0 = sload(p.ptr, kt), e1 = sload(p.ptr, kt + 1);
+  const int e0 = min(max(sload(p.ptr, kt), 0), p.nnz), e1 = min(max(sload(p.ptr, kt + 1), e0), p.nnz);
   const int n_half = 2 * (e1 - e0);
   // half tile i = half (i & 1) of list entry e0 + i / 2.  The list entry (query tile, causal
   // flag) of half tile i+1 is fetched one step before it is needed, so that no step starts by
@@ -484,7 +486,7 @@ __global__ __launch_bounds__(256, 2) void dq_kernel(const BwdParams p) {
   auto v_rsrc = [&](int kt) { return make_rsrc(vbase + (int64_t)kt * kTile * v_stride, v_extent); };
   auto ktile = [&](int e) { return min(max(sload(p.idx, e), 0), p.n_ktiles - 1); };
 
-  const int e0 = sload(p.ptr, qt), e1 = sload(p.ptr, qt + 1);
+  const int e0 = min(max(sload(p.ptr, qt), 0), p.nnz), e1 = min(max(sload(p.ptr, qt + 1), e0), p.nnz);
   int kt = e0 < e1 ? ktile(e0) : 0;
   if (e0 < e1) {
     dma_half_tile_buf<4>(sKA, k_rsrc(kt), koff, 0, wave);
@@ -534,11 +536,13 @@ __global__ __launch_bounds__(256, 2) void dq_kernel(const BwdParams p) {
 }
 
 static int fill_common(BwdParams& p, const void* q, const void* k, const void* v, const void* dout,
-                       const float* lse, const float* delta, int batch, int n_heads, int n_qtiles,
-                       int n_ktiles, int head_dim, const int64_t* qs, const int64_t* ks,
+                       const float* lse, const float* delta, const int32_t* idx, const uint8_t* flag,
+                       int batch, int n_heads, int n_qtiles,
+                       int n_ktiles, int nnz, int head_dim, const int64_t* qs, const int64_t* ks,
                        const int64_t* vs, const int64_t* ds, float softmax_scale) {
   if (!q || !k || !v || !dout || !lse || !delta || !qs || !ks || !vs || !ds) return UA_ERR_NULL;
-  if (batch <= 0 || n_heads <= 0 || n_qtiles <= 0 || n_ktiles <= 0) return UA_ERR_SHAPE;
+  if (batch <= 0 || n_heads <= 0 || n_qtiles <= 0 || n_ktiles <= 0 || nnz < 0) return UA_ERR_SHAPE;
+  if (nnz > 0 && (!idx || !flag)) return UA_ERR_NULL;          // only an empty list may leave them out
   if ((int64_t)batch * n_heads * n_qtiles > INT32_MAX || (int64_t)batch * n_heads * n_ktiles > INT32_MAX)
     return UA_ERR_SHAPE;
   if (head_dim != kHeadDim || !(softmax_scale > 0.f)) return UA_ERR_UNSUPPORTED;
@@ -548,7 +552,7 @@ static int fill_common(BwdParams& p, const void* q, const void* k, const void* v
     if (st[1] > (INT32_MAX >> 9)) return UA_ERR_SHAPE;
   p.q = (const bf16*)q; p.k = (const bf16*)k; p.v = (const bf16*)v; p.dout = (const bf16*)dout;
   p.lse = lse; p.delta = delta;
-  p.batch = batch; p.n_heads = n_heads; p.n_qtiles = n_qtiles; p.n_ktiles = n_ktiles;
+  p.batch = batch; p.n_heads = n_heads; p.n_qtiles = n_qtiles; p.n_ktiles = n_ktiles; p.nnz = nnz;
   p.qs = {qs[0], qs[1], qs[2]}; p.ks = {ks[0], ks[1], ks[2]};
   p.vs = {vs[0], vs[1], vs[2]}; p.ds = {ds[0], ds[1], ds[2]};
   p.scale = softmax_scale; p.scale_log2 = softmax_scale * kLog2e;
@@ -563,14 +567,14 @@ extern "C" int ua_bsa_bwd_dkdv(const void* q, const void* k, const void* v, cons
                                const float* lse, const float* delta, void* dk, void* dv,
                                const int32_t* col_ptr, const int32_t* row_idx, const uint8_t* cflag,
                                const int32_t* k_order,
-                               int batch, int n_heads, int n_qtiles, int n_ktiles, int head_dim,
+                               int batch, int n_heads, int n_qtiles, int n_ktiles, int nnz, int head_dim,
                                const int64_t* q_strides, const int64_t* k_strides, const int64_t* v_strides,
                                const int64_t* do_strides, const int64_t* dk_strides, const int64_t* dv_strides,
                                float softmax_scale, void* stream) {
   using namespace ua;
   BwdParams p;
-  if (int rc = fill_common(p, q, k, v, dout, lse, delta, batch, n_heads, n_qtiles, n_ktiles, head_dim,
-                           q_strides, k_strides, v_strides, do_strides, softmax_scale)) return rc;
+  if (int rc = fill_common(p, q, k, v, dout, lse, delta, row_idx, cflag, batch, n_heads, n_qtiles, n_ktiles, nnz,
+                           head_dim, q_strides, k_strides, v_strides, do_strides, softmax_scale)) return rc;
   if (!dk || !dv || !col_ptr || !k_order || !dk_strides || !dv_strides) return UA_ERR_NULL;
   if (!aligned16(dk) || !aligned16(dv) || !strides_ok(dk_strides) || !strides_ok(dv_strides)) return UA_ERR_ALIGN;
   p.out0 = (bf16*)dk; p.out1 = (bf16*)dv;
@@ -585,14 +589,14 @@ extern "C" int ua_bsa_bwd_dq(const void* q, const void* k, const void* v, const 
                              const float* lse, const float* delta, void* dq,
                              const int32_t* row_ptr, const int32_t* col_idx, const uint8_t* flag,
                              const int32_t* q_order,
-                             int batch, int n_heads, int n_qtiles, int n_ktiles, int head_dim,
+                             int batch, int n_heads, int n_qtiles, int n_ktiles, int nnz, int head_dim,
                              const int64_t* q_strides, const int64_t* k_strides, const int64_t* v_strides,
                              const int64_t* do_strides, const int64_t* dq_strides,
                              float softmax_scale, void* stream) {
   using namespace ua;
   BwdParams p;
-  if (int rc = fill_common(p, q, k, v, dout, lse, delta, batch, n_heads, n_qtiles, n_ktiles, head_dim,
-                           q_strides, k_strides, v_strides, do_strides, softmax_scale)) return rc;
+  if (int rc = fill_common(p, q, k, v, dout, lse, delta, col_idx, flag, batch, n_heads, n_qtiles, n_ktiles, nnz,
+                           head_dim, q_strides, k_strides, v_strides, do_strides, softmax_scale)) return rc;
   if (!dq || !row_ptr || !q_order || !dq_strides) return UA_ERR_NULL;
   if (!aligned16(dq) || !strides_ok(dq_strides)) return UA_ERR_ALIGN;
   p.out0 = (bf16*)dq; p.out1 = nullptr;

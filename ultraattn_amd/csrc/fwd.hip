@@ -18,7 +18,7 @@ namespace ua {
 struct FwdParams {
   const bf16* q; const bf16* k; const bf16* v; bf16* o; float* lse;
   const int32_t* row_ptr; const int32_t* col_idx; const uint8_t* flag; const int32_t* q_order;
-  int batch, n_heads, n_qtiles, n_ktiles;
+  int batch, n_heads, n_qtiles, n_ktiles, nnz;
   Strides3 qs, ks, vs, os;
   float scale_log2;      // softmax_scale * log2(e)
   int heads_per_xcd;     // batch*n_heads / 8 when divisible, else 0
@@ -148,7 +148,8 @@ __global__ __launch_bounds__(256, 2) void fwd_kernel(const FwdParams p) {
 
   const bf16* kbase = p.k + b * p.ks.b + h * p.ks.h;
   const bf16* vbase = p.v + b * p.vs.b + h * p.vs.h;
-  const int e0 = sload(p.row_ptr, qt), e1 = sload(p.row_ptr, qt + 1);
+  // list bounds are clamped to the arrays' extent: an inconsistent row_ptr cannot read beyond them
+  const int e0 = min(max(sload(p.row_ptr, qt), 0), p.nnz), e1 = min(max(sload(p.row_ptr, qt + 1), e0), p.nnz);
   const int k_stride = (int)p.ks.s, v_stride = (int)p.vs.s;
   int koff[4], voff[4];
   dma_voffsets<lds_off_k, 4>(koff, k_stride, wave, lane);
@@ -228,13 +229,14 @@ __global__ __launch_bounds__(256, 2) void fwd_kernel(const FwdParams p) {
 extern "C" int ua_bsa_fwd(const void* q, const void* k, const void* v, void* o, float* lse,
                           const int32_t* row_ptr, const int32_t* col_idx, const uint8_t* flag,
                           const int32_t* q_order,
-                          int batch, int n_heads, int n_qtiles, int n_ktiles, int head_dim,
+                          int batch, int n_heads, int n_qtiles, int n_ktiles, int nnz, int head_dim,
                           const int64_t* q_strides, const int64_t* k_strides, const int64_t* v_strides,
                           const int64_t* o_strides, float softmax_scale, void* stream) {
   using namespace ua;
   if (!q || !k || !v || !o || !lse || !row_ptr || !q_order || !q_strides || !k_strides || !v_strides || !o_strides)
     return UA_ERR_NULL;
-  if (batch <= 0 || n_heads <= 0 || n_qtiles <= 0 || n_ktiles <= 0) return UA_ERR_SHAPE;
+  if (batch <= 0 || n_heads <= 0 || n_qtiles <= 0 || n_ktiles <= 0 || nnz < 0) return UA_ERR_SHAPE;
+  if (nnz > 0 && (!col_idx || !flag)) return UA_ERR_NULL;      // only an empty list may leave them out
   if ((int64_t)batch * n_heads * n_qtiles > INT32_MAX) return UA_ERR_SHAPE;
   if (head_dim != kHeadDim || !(softmax_scale > 0.f)) return UA_ERR_UNSUPPORTED;
   if (!aligned16(q) || !aligned16(k) || !aligned16(v) || !aligned16(o)) return UA_ERR_ALIGN;
@@ -245,7 +247,7 @@ extern "C" int ua_bsa_fwd(const void* q, const void* k, const void* v, void* o, 
   FwdParams p;
   p.q = (const bf16*)q; p.k = (const bf16*)k; p.v = (const bf16*)v; p.o = (bf16*)o; p.lse = lse;
   p.row_ptr = row_ptr; p.col_idx = col_idx; p.flag = flag; p.q_order = q_order;
-  p.batch = batch; p.n_heads = n_heads; p.n_qtiles = n_qtiles; p.n_ktiles = n_ktiles;
+  p.batch = batch; p.n_heads = n_heads; p.n_qtiles = n_qtiles; p.n_ktiles = n_ktiles; p.nnz = nnz;
   p.qs = {q_strides[0], q_strides[1], q_strides[2]};
   p.ks = {k_strides[0], k_strides[1], k_strides[2]};
   p.vs = {v_strides[0], v_strides[1], v_strides[2]};

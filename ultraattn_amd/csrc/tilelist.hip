@@ -13,7 +13,7 @@ namespace ua {
 // type of tile (qt, kt): 0 empty, 1 full, 2 causal
 __host__ __device__ __forceinline__ int tile_type(const uint8_t* mask, int nkb, int rate, int qt, int kt) {
   const int t = mask[(int64_t)(qt / rate) * nkb + kt / rate];
-  if (t != 2) return t;
+  if (t != 2) return t == 1 ? 1 : 0;
   const int a = qt % rate, b = kt % rate;
   return a == b ? 2 : (a > b ? 1 : 0);
 }
@@ -93,6 +93,23 @@ __global__ __launch_bounds__(64 * kWavesPerGroup) void tl_count_kernel(const uin
   for (int i = lane; i < ln.n_blocks; i += 64) n += tiles_of_block(ln, mask[ln.base + i * ln.step], rate);
   n = wave_sum(n);
   if (lane == 0) (ln.is_row ? qcnt : kcnt)[ln.id] = n;
+}
+
+// check: a single workgroup counts the mask entries that are not a Block_Type (> 2); the
+// builder treats them as EMPTY, and the count lets the caller detect them after the stream
+// has been synchronised (the host builder returns UA_ERR_MASK for the same input).
+__global__ __launch_bounds__(1024) void tl_check_kernel(const uint8_t* mask, int64_t n, int32_t* n_invalid) {
+  __shared__ int32_t part[16];
+  int bad = 0;
+  for (int64_t i = threadIdx.x; i < n; i += 1024) bad += mask[i] > 2;
+  bad = wave_sum(bad);
+  if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = bad;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    int s = 0;
+    for (int i = 0; i < 16; ++i) s += part[i];
+    *n_invalid = s;
+  }
 }
 
 // scan: a single workgroup turns counts into exclusive prefix sums.
@@ -244,6 +261,7 @@ extern "C" int ua_tilelist_build_device(const uint8_t* block_mask, int n_qblocks
   hipStream_t st = (hipStream_t)stream;
   int32_t* qcnt = work;
   int32_t* kcnt = work + nqt + 1;
+  hipLaunchKernelGGL(tl_check_kernel, dim3(1), dim3(1024), 0, st, block_mask, (int64_t)n_qblocks * n_kblocks, work + nqt + nkt + 2);
   const int blocks = (nqt + nkt + kWavesPerGroup - 1) / kWavesPerGroup;
   hipLaunchKernelGGL(tl_count_kernel, dim3(blocks), dim3(64 * kWavesPerGroup), 0, st, block_mask, n_qblocks, n_kblocks, rate, qcnt, kcnt);
   hipLaunchKernelGGL(tl_scan_kernel, dim3(1), dim3(1024), 0, st, (const int32_t*)qcnt, nqt, row_ptr);

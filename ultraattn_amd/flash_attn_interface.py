@@ -20,7 +20,8 @@ from .tilelist import TILE, TileList, build_tile_list
 def _dense_tiles(n_qtiles: int, n_ktiles: int, causal: bool) -> TileList:
     m = np.ones((n_qtiles, n_ktiles), np.uint8)
     if causal:
-        # flash-attn aligns the causal diagonal to the bottom-right corner when Sq != Skv
+        # flash-attn (2.1 and later) aligns the causal diagonal to the bottom-right corner when
+        # Sq != Skv: query i sees key j iff j <= i + Skv - Sq; rows above the first key see nothing
         off = n_ktiles - n_qtiles
         i = np.arange(n_qtiles)[:, None] + off
         j = np.arange(n_ktiles)[None, :]
@@ -54,7 +55,7 @@ def _flash_attn_forward(q, k, v, dropout_p, softmax_scale, causal, window_size=(
 def _flash_attn_backward(dout, q, k, v, out, softmax_lse, dq, dk, dv, dropout_p, softmax_scale, causal,
                          window_size=(-1, -1), alibi_slopes=None, deterministic=False, rng_state=None,
                          softmax_d: Optional[torch.Tensor] = None):
-    """Writes dq, dk, dv in place; returns (dq, dk, dv, softmax_d).  With ``softmax_d`` given
+    """Writes dq, dk, dv in place (allocates the ones passed as None); returns (dq, dk, dv, softmax_d).  With ``softmax_d`` given
     ``out`` is ignored (the reference passes a dummy, ``orchestrated_attn_impl.py:583``).
     The kernels are deterministic regardless of ``deterministic``."""
     _check_unsupported(dropout_p, window_size, alibi_slopes)
@@ -64,5 +65,6 @@ def _flash_attn_backward(dout, q, k, v, out, softmax_lse, dq, dk, dv, dropout_p,
     if softmax_d is None:
         from .ops import softmax_delta
         softmax_d = softmax_delta(out, dout)
-    bsa_bwd(dout, q, k, v, None, softmax_lse, tiles, softmax_scale, dq=dq, dk=dk, dv=dv, softmax_d=softmax_d)
+    dq, dk, dv = bsa_bwd(dout, q, k, v, None, softmax_lse, tiles, softmax_scale, dq=dq, dk=dk, dv=dv,
+                         softmax_d=softmax_d)
     return dq, dk, dv, softmax_d

@@ -81,7 +81,7 @@ def bsa_fwd(q, k, v, tiles, softmax_scale: Optional[float] = None, causal: bool 
         st = torch.cuda.current_stream().cuda_stream
         rc = lib.ua_bsa_fwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), lse.data_ptr(),
                             d["row_ptr"].data_ptr(), d["col_idx"].data_ptr(), d["flag"].data_ptr(),
-                            d["q_order"].data_ptr(), B, Nh, tl.n_qtiles, tl.n_ktiles, D,
+                            d["q_order"].data_ptr(), B, Nh, tl.n_qtiles, tl.n_ktiles, tl.nnz, D,
                             _lib.strides3(q), _lib.strides3(k), _lib.strides3(v), _lib.strides3(out),
                             float(softmax_scale), st)
     _lib.check(rc, "ua_bsa_fwd")
@@ -142,14 +142,14 @@ def bsa_bwd(dout, q, k, v, out, lse, tiles, softmax_scale: Optional[float] = Non
         rc = lib.ua_bsa_bwd_dkdv(q.data_ptr(), k.data_ptr(), v.data_ptr(), dout.data_ptr(), lse.data_ptr(),
                                  softmax_d.data_ptr(), dk.data_ptr(), dv.data_ptr(),
                                  d["col_ptr"].data_ptr(), d["row_idx"].data_ptr(), d["cflag"].data_ptr(),
-                                 d["k_order"].data_ptr(), B, Nh, tl.n_qtiles, tl.n_ktiles, D,
+                                 d["k_order"].data_ptr(), B, Nh, tl.n_qtiles, tl.n_ktiles, tl.nnz, D,
                                  _lib.strides3(q), _lib.strides3(k), _lib.strides3(v), _lib.strides3(dout),
                                  _lib.strides3(dk), _lib.strides3(dv), float(softmax_scale), st)
         _lib.check(rc, "ua_bsa_bwd_dkdv")
         rc = lib.ua_bsa_bwd_dq(q.data_ptr(), k.data_ptr(), v.data_ptr(), dout.data_ptr(), lse.data_ptr(),
                                softmax_d.data_ptr(), dq.data_ptr(),
                                d["row_ptr"].data_ptr(), d["col_idx"].data_ptr(), d["flag"].data_ptr(),
-                               d["q_order"].data_ptr(), B, Nh, tl.n_qtiles, tl.n_ktiles, D,
+                               d["q_order"].data_ptr(), B, Nh, tl.n_qtiles, tl.n_ktiles, tl.nnz, D,
                                _lib.strides3(q), _lib.strides3(k), _lib.strides3(v), _lib.strides3(dout),
                                _lib.strides3(dq), float(softmax_scale), st)
         _lib.check(rc, "ua_bsa_bwd_dq")

@@ -104,29 +104,39 @@ class InputRowBwd:
         return softmax_delta(out, self.dO, delta=self.D)
 
 
-class OutputRowBwd:
+class _Fp32Accumulated:
+    """``reduce`` for gradient packs: the running sum is kept in fp32 beside the bf16 pack (the
+    accumulation the reference specifies, ``ring_flash_attn/ring_flash_attn.py:110-118``: partial
+    gradients are added into fp32 buffers and cast once), and ``data`` always holds its bf16
+    rounding.  Summing in bf16 instead loses about half a bit per partial."""
+    data: torch.Tensor
+    _acc = None
+
+    def reduce(self, other) -> None:
+        if self._acc is None:
+            self._acc = self.data.to(FULL_DTYPE)
+        self._acc.add_(other.data)            # bf16 -> fp32 promotion happens inside the add
+        self.data.copy_(self._acc)
+
+
+class OutputRowBwd(_Fp32Accumulated):
     """``Output_Row_Bwd`` (``orchestrated_attn/utils.py:237-262``): data = dQ; ``reduce`` is the
-    accumulation the reference leaves commented out (``:262``)."""
+    accumulation the reference leaves commented out (``:262``), done in fp32."""
 
     def __init__(self, buf: torch.Tensor, q_shape: Tuple[int, int, int, int]):
         self.data = _take(buf, 0, math.prod(q_shape))
         self.dQ = self.data.view(q_shape)
 
-    def reduce(self, other: "OutputRowBwd") -> None:
-        self.data.add_(other.data)
 
-
-class OutputColBwd:
-    """``Output_Col_Bwd`` (``orchestrated_attn/utils.py:264-298``): data = [dK | dV]."""
+class OutputColBwd(_Fp32Accumulated):
+    """``Output_Col_Bwd`` (``orchestrated_attn/utils.py:264-298``): data = [dK | dV]; ``reduce``
+    (``:296-298``) accumulates in fp32."""
 
     def __init__(self, buf: torch.Tensor, k_shape: Tuple[int, int, int, int]):
         n = math.prod(k_shape)
         self.data = _take(buf, 0, 2 * n)
         self.dK = self.data[:n].view(k_shape)
         self.dV = self.data[n:].view(k_shape)
-
-    def reduce(self, other: "OutputColBwd") -> None:
-        self.data.add_(other.data)
 
 
 def _permute_cols(entry: str, src: torch.Tensor, n_chunks: int, k_shape, out: torch.Tensor = None) -> torch.Tensor:

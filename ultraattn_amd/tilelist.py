@@ -91,11 +91,12 @@ def build_tile_list(block_mask, block: int = 512, tile: int = TILE, causal: bool
     return TileList(n_qtiles=nqt, n_ktiles=nkt, **arrs)
 
 
-def build_tile_list_device(block_mask_dev, block: int = 512, nnz: Optional[int] = None):
+def build_tile_list_device(block_mask_dev, block: int = 512, nnz: Optional[int] = None, check: bool = False):
     """Device-side builder: ``block_mask_dev`` is a uint8 CUDA tensor [n_qblocks, n_kblocks]
     (values 0/1/2, causal rule already applied).  Returns a dict of device tensors with the
     same contents as ``build_tile_list(...).on(device)``.  ``nnz`` (from a host-side size
-    query) trims the arrays; without it they are sized to the upper bound."""
+    query) trims the arrays; without it they are sized to the upper bound.  ``check`` reads back
+    the builder's count of invalid mask entries (this synchronises) and raises if it is not 0."""
     import torch
     m = block_mask_dev
     if m.dtype != torch.uint8 or m.dim() != 2 or not m.is_cuda or not m.is_contiguous():
@@ -111,13 +112,15 @@ def build_tile_list_device(block_mask_dev, block: int = 512, nnz: Optional[int] 
     out = dict(row_ptr=torch.empty(nqt + 1, **i32), col_idx=torch.empty(alloc, **i32), flag=torch.empty(alloc, **u8),
                col_ptr=torch.empty(nkt + 1, **i32), row_idx=torch.empty(alloc, **i32), cflag=torch.empty(alloc, **u8),
                q_order=torch.empty(nqt, **i32), k_order=torch.empty(nkt, **i32))
-    work = torch.empty(nqt + nkt + 2, **i32)
+    work = torch.empty(nqt + nkt + 3, **i32)
     lib = _lib.load()
     with torch.cuda.device(dev):
         st = torch.cuda.current_stream().cuda_stream
         _lib.check(lib.ua_tilelist_build_device(m.data_ptr(), nqb, nkb, rate,
                                                 *[out[n].data_ptr() for n in _HOST_FIELDS],
                                                 work.data_ptr(), st), "ua_tilelist_build_device")
+    if check and int(work[-1].item()) != 0:
+        raise ValueError(f"block mask holds {int(work[-1].item())} entries other than 0 (EMPTY), 1 (FULL), 2 (CAUSAL)")
     for n in ("col_idx", "flag", "row_idx", "cflag"):
         out[n] = out[n][:cap]
     return out
