@@ -135,6 +135,24 @@ int ua_bsa_bwd_dq(const void *q, const void *k, const void *v, const void *dout,
 int ua_merge(const void *const *o_parts, const float *const *lse_parts, int n_parts,
              void *o, float *lse, int batch, int seqlen, int n_heads, int head_dim, void *stream);
 
+/* In-place form of one `update_out_and_lse(out, lse, block_out, block_lse, slice_=None)` step
+ * (ring_flash_attn/utils.py:78-99, called with a row slice at
+ * hierarchy_attn/hierarchy_attn_impl.py:75-81): new_lse = logaddexp(lse, block_lse),
+ * new_out = exp(lse - new_lse) out + exp(block_lse - new_lse) block_out, max-stabilised.
+ * Every tensor is addressed through (batch, token, head) ELEMENT strides: rows
+ * [batch, n_rows, n_heads, 128] with head_dim contiguous (a row range of a larger tensor is a
+ * pointer offset), statistics fp32 in either the reference's running layout [B, S, Nh, 1]
+ * (strides S*Nh, Nh, 1) or the kernels' [B, Nh, S] (strides Nh*S, 1, S).  `*_is_fp32` select
+ * fp32 or bf16 rows (the reference's running `out` turns fp32 after its first update).
+ * new_out / new_lse may alias out / lse (the slice_ path) or be separate buffers.  Row strides
+ * must keep rows 16-byte aligned.                                                          */
+int ua_merge_update(const void *out, const float *lse, const void *block_out, const float *block_lse,
+                    void *new_out, float *new_lse, int batch, int n_rows, int n_heads, int head_dim,
+                    int out_is_fp32, int block_is_fp32, int new_is_fp32,
+                    const int64_t *out_strides, const int64_t *lse_strides,
+                    const int64_t *block_out_strides, const int64_t *block_lse_strides,
+                    const int64_t *new_out_strides, const int64_t *new_lse_strides, void *stream);
+
 /* ---- column-buffer layout changes around a fused rectangle -----------------------------------
  * Replace the two torch transpose+contiguous copies of the X x Y path:
  *   ua_cols_gather : buf.view(Y,2,B,Skv,Nh,D).transpose(0,1).transpose(1,2).flatten(2,3).contiguous()

@@ -21,7 +21,7 @@ def declared_symbols():
 
 def test_header_symbols_are_exported(lib):
     names = declared_symbols()
-    assert {"ua_bsa_fwd", "ua_bsa_bwd_dkdv", "ua_bsa_bwd_dq", "ua_bsa_bwd_delta", "ua_merge",
+    assert {"ua_bsa_fwd", "ua_bsa_bwd_dkdv", "ua_bsa_bwd_dq", "ua_bsa_bwd_delta", "ua_merge", "ua_merge_update",
             "ua_tilelist_build", "ua_tilelist_size", "ua_tilelist_build_device", "ua_strerror",
             "ua_version"} <= set(names)
     assert "ua_probe_mfma" not in names, "bench-only diagnostics stay out of the product ABI"

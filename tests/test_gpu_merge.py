@@ -95,3 +95,65 @@ def test_kernel_tiles_plus_merge_equal_single_launch(cfg):
     torch.cuda.synchronize()
     assert (o.float() - whole_o.float()).abs().max().item() <= ATOL_O
     assert lse_rel_err(l, whole_lse) <= RTOL_LSE
+
+
+# ---- update_out_and_lse drop-in (ring_flash_attn/utils.py:78-99) ---------------------------------
+
+def _ring_inputs(B, S, Nh, seed, n_blocks=3):
+    g = torch.Generator().manual_seed(seed)
+    outs = [torch.randn(B, S, Nh, 128, generator=g).to(torch.bfloat16) for _ in range(n_blocks)]
+    lses = [torch.randn(B, Nh, S, generator=g) * 3.0 for _ in range(n_blocks)]
+    return outs, lses
+
+
+@pytest.mark.parametrize("shape", [(1, 256, 4), (2, 48, 3), (1, 37, 5)])
+def test_update_out_and_lse_chain_vs_oracle(shape):
+    """The executors' accumulation loop (hierarchy_attn_impl.py:64-81): first partial initialises,
+    the second is folded into all rows, the third into the second half of the rows only
+    (slice_).  Same calls on the oracle (CPU, the reference's literal formula) and on the GPU."""
+    B, S, Nh = shape
+    outs, lses = _ring_inputs(B, S, Nh, seed=S)
+    half = S // 2
+    sl = (slice(None), slice(half, None))
+    ro, rl = None, None
+    ro, rl = ao.update_out_and_lse(ro, rl, outs[0], lses[0])
+    ro, rl = ao.update_out_and_lse(ro, rl, outs[1], lses[1])
+    ro, rl = ao.update_out_and_lse(ro, rl, outs[2][:, half:], lses[2][:, :, half:].contiguous(), slice_=sl)
+    d = lambda t: t.to(DEV)
+    o, l = None, None
+    o, l = ops.update_out_and_lse(o, l, d(outs[0]), d(lses[0]))
+    assert o.dtype == torch.bfloat16 and l.shape == (B, S, Nh, 1)             # as the reference: block_out itself
+    o, l = ops.update_out_and_lse(o, l, d(outs[1]), d(lses[1]))
+    assert o.dtype == ro.dtype == torch.float32 and l.shape == rl.shape == (B, S, Nh, 1)
+    before = o[:, :half].clone()
+    o2, l2 = ops.update_out_and_lse(o, l, d(outs[2][:, half:].contiguous()), d(lses[2][:, :, half:].contiguous()), slice_=sl)
+    torch.cuda.synchronize()
+    assert o2.data_ptr() == o.data_ptr() and l2.data_ptr() == l.data_ptr()     # slice_ updates in place
+    assert torch.equal(o[:, :half], before)                                    # rows outside the slice untouched
+    # fp32 rows and statistics on both sides: only the exp2/log2 hardware approximations differ
+    assert max_abs(o2, ro) <= 3e-5 and (l2.cpu() - rl).abs().max().item() <= 1e-5
+
+
+def test_update_out_and_lse_bf16_in_place_and_statistics_layouts():
+    """slice_ on a bf16 running output stays bf16 (assignment casts, utils.py:95), block_lse may
+    come as [B,S,Nh,1] (hierarchy_attn_impl.py:52) and -inf partials are the identity."""
+    B, S, Nh = 1, 64, 4
+    outs, lses = _ring_inputs(B, S, Nh, seed=3, n_blocks=2)
+    lses[1][0, 1, 5:9] = float("-inf")                    # block without keys on some rows
+    lses[0][0, 2, 20:24] = float("-inf")                  # running rows that have seen no key yet
+    lses[0][0, 3, 40] = lses[1][0, 3, 40] = float("-inf")  # neither has
+    run_o = outs[0].to(DEV)
+    run_l = lses[0].transpose(-2, -1).unsqueeze(-1).contiguous().to(DEV)          # [B,S,Nh,1]
+    blk_l = lses[1].transpose(-2, -1).unsqueeze(-1).contiguous().to(DEV)          # [B,S,Nh,1] as well
+    o, l = ops.update_out_and_lse(run_o, run_l, outs[1].to(DEV), blk_l, slice_=(slice(None), slice(None)))
+    torch.cuda.synchronize()
+    assert o.dtype == torch.bfloat16 and o.data_ptr() == run_o.data_ptr()
+    ro, rl = ao.merge_partials(outs, lses)
+    assert torch.isfinite(o).all()
+    assert max_abs(o, ro) <= ATOL_O and lse_rel_err(l.squeeze(-1).transpose(1, 2), rl) <= RTOL_LSE
+    assert (o[0, 40, 3] == 0).all() and torch.equal(o[0, 5:9, 1].cpu(), outs[0][0, 5:9, 1])
+    assert torch.equal(o[0, 20:24, 2].cpu(), outs[1][0, 20:24, 2])
+    with pytest.raises(RuntimeError):
+        ops.update_out_and_lse(None, None, outs[0].to(DEV), lses[0].to(DEV), slice_=(slice(None),))
+    with pytest.raises(ValueError):
+        ops.update_out_and_lse(run_o, run_l, outs[1][:, :32].to(DEV), blk_l)

@@ -23,6 +23,7 @@ SIGNATURES = {
     "ua_bsa_bwd_dq": (c_int, [c_void_p] * 11 + [c_int] * 6 + [_i64p] * 5 + [c_float, c_void_p]),
     "ua_merge": (c_int, [POINTER(c_void_p), POINTER(c_void_p), c_int, c_void_p, c_void_p,
                          c_int, c_int, c_int, c_int, c_void_p]),
+    "ua_merge_update": (c_int, [c_void_p] * 6 + [c_int] * 7 + [_i64p] * 6 + [c_void_p]),
     "ua_cols_gather": (c_int, [c_void_p, c_void_p, c_int, c_int, c_int64, c_void_p]),
     "ua_cols_scatter": (c_int, [c_void_p, c_void_p, c_int, c_int, c_int64, c_void_p]),
 }

@@ -185,3 +185,80 @@ def merge_partials(outs: Sequence[torch.Tensor], lses: Sequence[torch.Tensor],
         rc = lib.ua_merge(op, lp, P, out.data_ptr(), lse.data_ptr(), B, S, Nh, D, st)
     _lib.check(rc, "ua_merge")
     return out, lse
+
+
+def _strides_bsh(t: torch.Tensor, layout: str):
+    """(batch, token, head) element strides of a statistics tensor given as [B, S, Nh, 1]
+    ('bsh1') or [B, Nh, S] ('bhs'), or of a [B, S, Nh, D] row tensor ('rows')."""
+    if layout == "bhs":
+        return (ctypes.c_int64 * 3)(t.stride(0), t.stride(2), t.stride(1))
+    return (ctypes.c_int64 * 3)(t.stride(0), t.stride(1), t.stride(2))
+
+
+def _stat_layout(t: torch.Tensor, B: int, S: int, Nh: int, name: str) -> str:
+    if t.dtype != torch.float32 or not t.is_cuda:
+        raise TypeError(f"{name} must be a float32 CUDA tensor")
+    if t.dim() == 4 and tuple(t.shape) == (B, S, Nh, 1):
+        return "bsh1"
+    if t.dim() == 3 and tuple(t.shape) == (B, Nh, S):
+        return "bhs"
+    raise ValueError(f"{name} must be [B, S, Nh, 1] or [B, Nh, S] = ({B}, {S}, {Nh}), got {tuple(t.shape)}")
+
+
+def _check_rows(name: str, t: torch.Tensor):
+    if not t.is_cuda or t.dtype not in (torch.bfloat16, torch.float32):
+        raise TypeError(f"{name} must be a bfloat16 or float32 CUDA tensor")
+    if t.dim() != 4 or t.shape[-1] != HEAD_DIM or t.stride(-1) != 1:
+        raise ValueError(f"{name} must be [B, S, Nh, {HEAD_DIM}] with a contiguous last axis, got {tuple(t.shape)}")
+
+
+def update_out_and_lse(out: Optional[torch.Tensor], lse: Optional[torch.Tensor], block_out: torch.Tensor,
+                       block_lse: torch.Tensor, slice_=None) -> Tuple[torch.Tensor, torch.Tensor]:
+    """Drop-in for ``update_out_and_lse`` of the ring / hierarchy executors
+    (``ring_flash_attn/utils.py:78-99``; call sites ``hierarchy_attn/hierarchy_attn_impl.py:64-81``):
+    folds one more partial ``(block_out [B,Sb,Nh,D], block_lse [B,Nh,Sb])`` into the running
+    ``(out [B,S,Nh,D], lse [B,S,Nh,1])`` and returns the pair.
+
+    * first call (``out is None``): returns ``block_out`` and ``block_lse`` as ``[B,S,Nh,1]``, as the
+      reference does (``slice_`` is then an error);
+    * ``slice_`` (an index for both ``out`` and ``lse``, e.g. ``(slice(None), slice(S//2, None))``):
+      the rows it selects are updated in place, in ``out``'s dtype;
+    * otherwise new tensors are returned and ``out`` is fp32, which is what the reference's
+      expression yields (fp32 statistics times bf16 rows).
+    One kernel (``ua_merge_update``) in place of the reference's eight element-wise launches; the
+    arithmetic is max-stabilised and treats ``lse = -inf`` as "no keys", which the literal formula
+    does not (it agrees with it on every input where that one is finite).  ``block_lse`` may also
+    come as ``[B,Sb,Nh,1]`` (the hierarchy executor's ``forward`` closure, ``:40-53``)."""
+    if out is None:
+        if slice_ is not None:
+            raise RuntimeError("first update_out_and_lse should not pass slice_ args")
+        if block_lse.dim() == 3:
+            block_lse = block_lse.transpose(-2, -1).unsqueeze(dim=-1)
+        return block_out, block_lse
+    _check_rows("out", out)
+    _check_rows("block_out", block_out)
+    if slice_ is not None:
+        tgt_out, tgt_lse = out[slice_], lse[slice_]
+        new_out, new_lse = tgt_out, tgt_lse                    # views: written in place
+    else:
+        tgt_out, tgt_lse = out, lse
+        new_out = torch.empty(out.shape, dtype=torch.float32, device=out.device)
+        new_lse = torch.empty(lse.shape, dtype=torch.float32, device=out.device)
+    _check_rows("out[slice_]", tgt_out)
+    B, S, Nh, D = tgt_out.shape
+    if tuple(block_out.shape) != (B, S, Nh, D):
+        raise ValueError(f"block_out is {tuple(block_out.shape)}, the rows to update are {(B, S, Nh, D)}")
+    l_lay = _stat_layout(tgt_lse, B, S, Nh, "lse")
+    b_lay = _stat_layout(block_lse, B, S, Nh, "block_lse")
+    lib = _lib.load()
+    with torch.cuda.device(out.device):
+        st = torch.cuda.current_stream().cuda_stream
+        rc = lib.ua_merge_update(tgt_out.data_ptr(), tgt_lse.data_ptr(), block_out.data_ptr(), block_lse.data_ptr(),
+                                 new_out.data_ptr(), new_lse.data_ptr(), B, S, Nh, D,
+                                 int(tgt_out.dtype == torch.float32), int(block_out.dtype == torch.float32),
+                                 int(new_out.dtype == torch.float32),
+                                 _strides_bsh(tgt_out, "rows"), _strides_bsh(tgt_lse, l_lay),
+                                 _strides_bsh(block_out, "rows"), _strides_bsh(block_lse, b_lay),
+                                 _strides_bsh(new_out, "rows"), _strides_bsh(new_lse, l_lay), st)
+    _lib.check(rc, "ua_merge_update")
+    return (out, lse) if slice_ is not None else (new_out, new_lse)
