@@ -247,21 +247,16 @@ extern "C" int ua_tilelist_build(const uint8_t* block_mask, int n_qblocks, int n
   return UA_OK;
 }
 
-extern "C" int ua_tilelist_build_device(const uint8_t* block_mask, int n_qblocks, int n_kblocks, int rate,
-                                        int32_t* row_ptr, int32_t* col_idx, uint8_t* flag,
-                                        int32_t* col_ptr, int32_t* row_idx, uint8_t* cflag,
-                                        int32_t* q_order, int32_t* k_order, int32_t* work, void* stream) {
-  using namespace ua;
-  if (!block_mask || !row_ptr || !col_idx || !flag || !col_ptr || !row_idx || !cflag || !q_order || !k_order || !work)
-    return UA_ERR_NULL;
-  if (n_qblocks <= 0 || n_kblocks <= 0 || rate <= 0) return UA_ERR_SHAPE;
-  if ((int64_t)n_qblocks * rate > (1 << 24) || (int64_t)n_kblocks * rate > (1 << 24)) return UA_ERR_SHAPE;
-  if (int rc = check_device()) return rc;
+namespace ua {
+
+static int build_device_impl(const uint8_t* block_mask, int n_qblocks, int n_kblocks, int rate,
+                             int32_t* row_ptr, int32_t* col_idx, uint8_t* flag,
+                             int32_t* col_ptr, int32_t* row_idx, uint8_t* cflag,
+                             int32_t* q_order, int32_t* k_order, int32_t* work, int32_t* n_invalid, hipStream_t st) {
   const int nqt = n_qblocks * rate, nkt = n_kblocks * rate;
-  hipStream_t st = (hipStream_t)stream;
   int32_t* qcnt = work;
   int32_t* kcnt = work + nqt + 1;
-  hipLaunchKernelGGL(tl_check_kernel, dim3(1), dim3(1024), 0, st, block_mask, (int64_t)n_qblocks * n_kblocks, work + nqt + nkt + 2);
+  hipLaunchKernelGGL(tl_check_kernel, dim3(1), dim3(1024), 0, st, block_mask, (int64_t)n_qblocks * n_kblocks, n_invalid);
   const int blocks = (nqt + nkt + kWavesPerGroup - 1) / kWavesPerGroup;
   hipLaunchKernelGGL(tl_count_kernel, dim3(blocks), dim3(64 * kWavesPerGroup), 0, st, block_mask, n_qblocks, n_kblocks, rate, qcnt, kcnt);
   hipLaunchKernelGGL(tl_scan_kernel, dim3(1), dim3(1024), 0, st, (const int32_t*)qcnt, nqt, row_ptr);
@@ -272,4 +267,29 @@ extern "C" int ua_tilelist_build_device(const uint8_t* block_mask, int n_qblocks
                      (const int32_t*)row_ptr, (const int32_t*)col_idx, nqt, q_order,
                      (const int32_t*)col_ptr, (const int32_t*)row_idx, nkt, k_order);
   return hipGetLastError() == hipSuccess ? UA_OK : UA_ERR_LAUNCH;
+}
+
+static int check_device_builder_args(const uint8_t* block_mask, int n_qblocks, int n_kblocks, int rate,
+                                     const void* row_ptr, const void* col_idx, const void* flag, const void* col_ptr,
+                                     const void* row_idx, const void* cflag, const void* q_order, const void* k_order) {
+  if (!block_mask || !row_ptr || !col_idx || !flag || !col_ptr || !row_idx || !cflag || !q_order || !k_order)
+    return UA_ERR_NULL;
+  if (n_qblocks <= 0 || n_kblocks <= 0 || rate <= 0) return UA_ERR_SHAPE;
+  if ((int64_t)n_qblocks * rate > (1 << 24) || (int64_t)n_kblocks * rate > (1 << 24)) return UA_ERR_SHAPE;
+  return check_device();
+}
+
+}  // namespace ua
+
+extern "C" int ua_tilelist_build_device(const uint8_t* block_mask, int n_qblocks, int n_kblocks, int rate,
+                                        int32_t* row_ptr, int32_t* col_idx, uint8_t* flag,
+                                        int32_t* col_ptr, int32_t* row_idx, uint8_t* cflag,
+                                        int32_t* q_order, int32_t* k_order, int32_t* work, void* stream) {
+  using namespace ua;
+  if (!work) return UA_ERR_NULL;
+  if (int rc = check_device_builder_args(block_mask, n_qblocks, n_kblocks, rate, row_ptr, col_idx, flag, col_ptr,
+                                         row_idx, cflag, q_order, k_order)) return rc;
+  const int nqt = n_qblocks * rate, nkt = n_kblocks * rate;
+  return build_device_impl(block_mask, n_qblocks, n_kblocks, rate, row_ptr, col_idx, flag, col_ptr, row_idx, cflag,
+                           q_order, k_order, work, work + nqt + nkt + 2, (hipStream_t)stream);
 }
