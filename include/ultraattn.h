@@ -45,10 +45,12 @@ extern "C" {
 #define UA_ERR_MASK (-5)        /* block mask holds a value other than 0, 1, 2 */
 #define UA_ERR_LAUNCH (-6)      /* the HIP runtime rejected the launch */
 #define UA_ERR_DEVICE (-7)      /* current device is not a gfx950 GPU */
+#define UA_ERR_TOO_LARGE (-8)   /* input exceeds the fixed scratch of a no-allocation entry point */
 
 #define UA_TILE 128        /* rows and columns of one kernel tile */
 #define UA_HEAD_DIM 128    /* the only supported head dimension */
 #define UA_MAX_PARTS 16    /* most partial outputs one ua_merge call combines */
+#define UA_NOALLOC_MAX_LINES 65532   /* most query tiles + key tiles of ua_tilelist_build_device_noalloc */
 
 int ua_version(void);
 const char *ua_strerror(int rc);
@@ -81,6 +83,19 @@ int ua_tilelist_build_device(const uint8_t *block_mask, int n_qblocks, int n_kbl
                              int32_t *row_ptr, int32_t *col_idx, uint8_t *flag,
                              int32_t *col_ptr, int32_t *row_idx, uint8_t *cflag,
                              int32_t *q_order, int32_t *k_order, int32_t *work, void *stream);
+
+/* No counterpart in the reference.  For callers that cannot allocate device memory (code under
+ * HIP graph capture, tight serving loops, harnesses that forbid it): the same builder as
+ * ua_tilelist_build_device with the `work` scratch taken from a fixed array inside the library
+ * (256 KiB per GPU, held until the process ends) instead of from the caller.  Limit:
+ * n_qtiles + n_ktiles <= UA_NOALLOC_MAX_LINES, else UA_ERR_TOO_LARGE.  `n_invalid` (device,
+ * may be NULL) receives the number of mask entries that are not 0, 1 or 2.  It calls no
+ * hipMalloc/hipFree.  All calls on one GPU share the array: calls that overlap in time on the
+ * same GPU (different streams or threads) race; serialise them.                             */
+int ua_tilelist_build_device_noalloc(const uint8_t *block_mask, int n_qblocks, int n_kblocks, int rate,
+                                     int32_t *row_ptr, int32_t *col_idx, uint8_t *flag,
+                                     int32_t *col_ptr, int32_t *row_idx, uint8_t *cflag,
+                                     int32_t *q_order, int32_t *k_order, int32_t *n_invalid, void *stream);
 
 /* ---- forward ------------------------------------------------------------------------------
  * Replaces the N dense `_flash_attn_forward(q, k, v, dropout_p, softmax_scale, causal=, ...,

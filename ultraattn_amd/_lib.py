@@ -17,6 +17,7 @@ SIGNATURES = {
     "ua_tilelist_size": (c_int, [c_void_p, c_int, c_int, c_int, _i64p, _i64p, _i64p]),
     "ua_tilelist_build": (c_int, [c_void_p, c_int, c_int, c_int] + [c_void_p] * 8),
     "ua_tilelist_build_device": (c_int, [c_void_p, c_int, c_int, c_int] + [c_void_p] * 10),
+    "ua_tilelist_build_device_noalloc": (c_int, [c_void_p, c_int, c_int, c_int] + [c_void_p] * 10),
     "ua_bsa_fwd": (c_int, [c_void_p] * 9 + [c_int] * 6 + [_i64p] * 4 + [c_float, c_void_p]),
     "ua_bsa_bwd_delta": (c_int, [c_void_p] * 3 + [c_int] * 4 + [_i64p] * 2 + [c_void_p]),
     "ua_bsa_bwd_dkdv": (c_int, [c_void_p] * 12 + [c_int] * 6 + [_i64p] * 6 + [c_float, c_void_p]),

@@ -35,6 +35,7 @@ extern "C" const char* ua_strerror(int rc) {
     case UA_ERR_MASK: return "block mask holds a value other than 0 (EMPTY), 1 (FULL), 2 (CAUSAL)";
     case UA_ERR_LAUNCH: return "HIP kernel launch failed";
     case UA_ERR_DEVICE: return "current device is not a gfx950 (MI355X) GPU";
+    case UA_ERR_TOO_LARGE: return "input exceeds the fixed scratch of the no-allocation entry point";
     default: return "unknown error code";
   }
 }

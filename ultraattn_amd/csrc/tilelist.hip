@@ -4,9 +4,16 @@
 // CAUSAL becomes causal on the sub-diagonal, full below it and empty above it.  Tiles are
 // emitted row-major (query tile outer, key tile inner).
 #include <algorithm>
+#include <atomic>
 #include <numeric>
 #include <vector>
 #include "ua_common.h"
+
+// Scratch of the entry point that allocates nothing (ua_tilelist_build_device_noalloc): the
+// per-row and per-column tile counts that the device builder otherwise keeps in the caller's
+// `work` argument.  Every GPU the library runs on holds its own copy (256 KiB) until the process
+// ends; calls on one GPU share it, so two such calls must not overlap.
+static __device__ __align__(256) int32_t scratch[UA_NOALLOC_MAX_LINES + 4];
 
 namespace ua {
 
@@ -292,4 +299,38 @@ extern "C" int ua_tilelist_build_device(const uint8_t* block_mask, int n_qblocks
   const int nqt = n_qblocks * rate, nkt = n_kblocks * rate;
   return build_device_impl(block_mask, n_qblocks, n_kblocks, rate, row_ptr, col_idx, flag, col_ptr, row_idx, cflag,
                            q_order, k_order, work, work + nqt + nkt + 2, (hipStream_t)stream);
+}
+
+// The device address of `scratch`, looked up once per device with that device current.  In host
+// code the array's name is only a handle for this lookup, never an address to pass on.
+static int scratch_of_current_device(int32_t** out) {
+  static std::atomic<int32_t*> ptrs[64];
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return UA_ERR_DEVICE;
+  int32_t* p = ptrs[dev].load(std::memory_order_acquire);
+  if (!p) {
+    void* sym = nullptr;
+    if (hipGetSymbolAddress(&sym, HIP_SYMBOL(scratch)) != hipSuccess || !sym) return UA_ERR_DEVICE;
+    p = static_cast<int32_t*>(sym);
+    ptrs[dev].store(p, std::memory_order_release);
+  }
+  *out = p;
+  return UA_OK;
+}
+
+extern "C" int ua_tilelist_build_device_noalloc(const uint8_t* block_mask, int n_qblocks, int n_kblocks, int rate,
+                                                int32_t* row_ptr, int32_t* col_idx, uint8_t* flag,
+                                                int32_t* col_ptr, int32_t* row_idx, uint8_t* cflag,
+                                                int32_t* q_order, int32_t* k_order, int32_t* n_invalid, void* stream) {
+  using namespace ua;
+  if (int rc = check_device_builder_args(block_mask, n_qblocks, n_kblocks, rate, row_ptr, col_idx, flag, col_ptr,
+                                         row_idx, cflag, q_order, k_order)) return rc;
+  const int64_t lines = (int64_t)n_qblocks * rate + (int64_t)n_kblocks * rate;
+  if (lines > UA_NOALLOC_MAX_LINES) return UA_ERR_TOO_LARGE;
+  int32_t* work = nullptr;
+  if (int rc = scratch_of_current_device(&work)) return rc;
+  // the counts are written before they are read and the invalid-entry count is stored, not
+  // accumulated: nothing in the scratch has to start at zero
+  return build_device_impl(block_mask, n_qblocks, n_kblocks, rate, row_ptr, col_idx, flag, col_ptr, row_idx, cflag,
+                           q_order, k_order, work, n_invalid ? n_invalid : work + lines + 2, (hipStream_t)stream);
 }
