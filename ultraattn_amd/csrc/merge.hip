@@ -1,7 +1,7 @@
 // LSE-weighted merge of partial attention outputs, and the backward's row statistic
 // delta = rowsum(dO * O).  Both are HBM-bandwidth bound streaming kernels.
 //
-// A workgroup owns kTok consecutive tokens of all heads.  The per-row statistics are laid out
+// A workgroup owns a few consecutive tokens (kTok, kMergeTok) of all heads.  The per-row statistics are laid out
 // [batch, head, token] while the rows themselves are [batch, token, head, 128]; the workgroup
 // first handles the statistics with token-contiguous (coalesced) accesses and parks the row
 // weights in LDS, then streams the rows as 16-byte vectors (16 lanes per 256-byte row).
@@ -9,7 +9,11 @@
 
 namespace ua {
 
-constexpr int kTok = 16;          // tokens per workgroup
+constexpr int kTok = 16;          // tokens per workgroup (delta, single update)
+// The merge runs best with many small workgroups: with 2 tokens x 32 heads a workgroup issues
+// all of its row loads in one step (4 x 16 bytes per thread and partial) and retires; the
+// device then streams 4 reads : 1 write at the rate a bare copy kernel of the same shape reaches.
+constexpr int kMergeTok = 2;
 constexpr int kMaxHeadsLds = 256; // rows per workgroup = kTok * n_heads <= 4096
 
 struct MergeParams {
@@ -21,12 +25,12 @@ struct MergeParams {
 
 template <int P>
 __global__ __launch_bounds__(256) void merge_kernel(const MergeParams p) {
-  extern __shared__ float w_lds[];              // [P][rows], rows = kTok * n_heads
+  extern __shared__ float w_lds[];              // [P][rows], rows = kMergeTok * n_heads
   const int tid = threadIdx.x;
-  const int tiles_per_batch = (p.seqlen + kTok - 1) / kTok;
+  const int tiles_per_batch = (p.seqlen + kMergeTok - 1) / kMergeTok;
   const int b = blockIdx.x / tiles_per_batch;
-  const int s0 = (blockIdx.x % tiles_per_batch) * kTok;
-  const int ntok = min(kTok, p.seqlen - s0);       // the last workgroup of a batch may be ragged
+  const int s0 = (blockIdx.x % tiles_per_batch) * kMergeTok;
+  const int ntok = min(kMergeTok, p.seqlen - s0);       // the last workgroup of a batch may be ragged
   const int rows = ntok * p.n_heads;
 
   // The rows are streamed as 16-byte chunks (chunk c = 8 bf16 of row c/16), kUnroll chunks per
@@ -51,8 +55,8 @@ __global__ __launch_bounds__(256) void merge_kernel(const MergeParams p) {
   load(tid);        // first step's rows are in flight while the statistics are handled
 
   // phase 1: one thread per (head, token): statistics, coalesced along the token axis
-  for (int t = tid; t < kTok * p.n_heads; t += 256) {
-    const int h = t / kTok, sl = t % kTok;
+  for (int t = tid; t < kMergeTok * p.n_heads; t += 256) {
+    const int h = t / kMergeTok, sl = t % kMergeTok;
     if (sl >= ntok) continue;
     const int64_t li = ((int64_t)b * p.n_heads + h) * p.seqlen + s0 + sl;
     float l[P];
@@ -119,19 +123,34 @@ __global__ __launch_bounds__(256) void delta_kernel(const DeltaParams p) {
   const int ntok = min(kTok, p.seqlen - s0);
   const int rows = ntok * p.n_heads;
   const int sub = tid & 15;
-  for (int row = tid >> 4; row < rows; row += 16) {
-    const int sl = row / p.n_heads, h = row % p.n_heads;
-    const int64_t s = s0 + sl;
-    const u32x4 a = *reinterpret_cast<const u32x4*>(p.o + b * p.os.b + s * p.os.s + h * p.os.h + sub * 8);
-    const u32x4 g = *reinterpret_cast<const u32x4*>(p.dout + b * p.ds.b + s * p.ds.s + h * p.ds.h + sub * 8);
-    float acc = 0.f;
+  // 16 lanes per row; kRows rows per thread and step so that 2 * kRows 16-byte loads are in flight
+  constexpr int kRows = 4;
+  for (int row0 = tid >> 4; row0 < rows; row0 += 16 * kRows) {
+    u32x4 a[kRows], g[kRows];
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      acc = fmaf(__uint_as_float(a[j] << 16), __uint_as_float(g[j] << 16), acc);
-      acc = fmaf(__uint_as_float(a[j] & 0xffff0000u), __uint_as_float(g[j] & 0xffff0000u), acc);
+    for (int u = 0; u < kRows; ++u) {
+      const int row = row0 + 16 * u;
+      if (row < rows) {
+        const int sl = row / p.n_heads, h = row % p.n_heads;
+        const int64_t s = s0 + sl;
+        a[u] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p.o + b * p.os.b + s * p.os.s + h * p.os.h + sub * 8));
+        g[u] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p.dout + b * p.ds.b + s * p.ds.s + h * p.ds.h + sub * 8));
+      }
     }
-    acc += __shfl_xor(acc, 1); acc += __shfl_xor(acc, 2); acc += __shfl_xor(acc, 4); acc += __shfl_xor(acc, 8);
-    if (sub == 0) d_lds[h * kTok + sl] = acc;
+#pragma unroll
+    for (int u = 0; u < kRows; ++u) {
+      const int row = row0 + 16 * u;
+      if (row >= rows) break;
+      const int sl = row / p.n_heads, h = row % p.n_heads;
+      float acc = 0.f;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        acc = fmaf(__uint_as_float(a[u][j] << 16), __uint_as_float(g[u][j] << 16), acc);
+        acc = fmaf(__uint_as_float(a[u][j] & 0xffff0000u), __uint_as_float(g[u][j] & 0xffff0000u), acc);
+      }
+      acc += __shfl_xor(acc, 1); acc += __shfl_xor(acc, 2); acc += __shfl_xor(acc, 4); acc += __shfl_xor(acc, 8);
+      if (sub == 0) d_lds[h * kTok + sl] = acc;
+    }
   }
   __syncthreads();
   for (int t = tid; t < kTok * p.n_heads; t += 256) {
@@ -242,7 +261,7 @@ extern "C" int ua_merge(const void* const* o_parts, const float* const* lse_part
   if (n_parts < 1 || n_parts > UA_MAX_PARTS) return UA_ERR_UNSUPPORTED;
   if (head_dim != kHeadDim) return UA_ERR_UNSUPPORTED;
   if (batch <= 0 || seqlen <= 0 || n_heads <= 0 || n_heads > kMaxHeadsLds) return UA_ERR_SHAPE;
-  if ((int64_t)batch * ((seqlen + kTok - 1) / kTok) > INT32_MAX) return UA_ERR_SHAPE;
+  if ((int64_t)batch * ((seqlen + kMergeTok - 1) / kMergeTok) > INT32_MAX) return UA_ERR_SHAPE;
   if (!aligned16(o)) return UA_ERR_ALIGN;
   MergeParams p;
   for (int i = 0; i < n_parts; ++i) {
@@ -254,8 +273,8 @@ extern "C" int ua_merge(const void* const* o_parts, const float* const* lse_part
   for (int i = n_parts; i < UA_MAX_PARTS; ++i) { p.o_parts[i] = nullptr; p.lse_parts[i] = nullptr; }
   p.o = (bf16*)o; p.lse = lse; p.n_parts = n_parts; p.seqlen = seqlen; p.n_heads = n_heads;
   if (int rc = check_device()) return rc;
-  const int blocks = batch * ((seqlen + kTok - 1) / kTok);
-  const size_t lds = (size_t)n_parts * kTok * n_heads * sizeof(float);
+  const int blocks = batch * ((seqlen + kMergeTok - 1) / kMergeTok);
+  const size_t lds = (size_t)n_parts * kMergeTok * n_heads * sizeof(float);
   if (lds > 65536) return UA_ERR_SHAPE;   // n_parts * n_heads <= 1024
   hipStream_t st = (hipStream_t)stream;
   switch (n_parts) {
