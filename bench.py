@@ -25,9 +25,46 @@ HBM_PEAK_GBPS = 8000.0            # MI355X HBM3E, published
 FLOP_PER_CLK_PER_CU = 4096        # dense bf16 MFMA, CDNA4
 
 
-# HBM bytes per launch of the dominant kernel, from profiles/hbm_traffic_<workload>.txt
-# (rocprofv3 --pmc FETCH_SIZE x 2.0 + WRITE_SIZE x 1.0, scaling explained there).
-TRAFFIC_BYTES = {("c3", "dkdv_kernel"): 41.84e9, ("c5", "fwd_kernel"): 10.85e9}
+# HBM-side bytes per launch, NOT measured by this run: constants copied from the rocprofv3 --pmc
+# summaries under profiles/ (FETCH_SIZE x 2.0 + WRITE_SIZE x 1.0, scaling explained there).  Every
+# roofline entry names the file its figure comes from; a kernel without a summary gets null.
+TRAFFIC_BYTES = {}        # filled from profiles/hbm_traffic_<workload>.txt by load_traffic()
+
+
+def load_traffic():
+    """Parse the 'HBM-side bytes per launch after scaling' tables of profiles/hbm_traffic_*.txt."""
+    import glob
+    import re
+    for path in sorted(glob.glob(os.path.join(ROOT, "profiles", "hbm_traffic_*.txt"))):
+        w = os.path.basename(path)[len("hbm_traffic_"):-4]
+        for m in re.finditer(r"^\s+ua::(\S+)\s+([0-9.]+) GB\s*$", open(path).read(), flags=re.M):
+            TRAFFIC_BYTES[(w, m.group(1))] = (float(m.group(2)) * 1e9, os.path.relpath(path, ROOT))
+
+
+def roof_entry(workload, kernel, bound, achieved, peak, unit, kernel_ms, algorithmic):
+    tr = TRAFFIC_BYTES.get((workload, kernel))
+    e = {"workload": workload, "kernel": kernel, "bound": bound, "achieved": achieved, "peak": peak, "unit": unit,
+         "frac": achieved / peak, "kernel_ms": kernel_ms,
+         "traffic": tr[0] if tr else None,
+         "traffic_source": (tr[1] + " (rocprofv3 --pmc, a constant from that file, not measured in this run)") if tr else None}
+    e["algorithmic_flops" if bound == "mfma" else "algorithmic_bytes"] = algorithmic
+    return e
+
+
+def attention_roofs(workload, res, peak):
+    """Roofline entries of the attention kernels of one workload result (algorithmic flops by the
+    reference's convention: forward F, dK/dV 4 of the backward's 5 GEMMs = 2.0 F, dQ 1 of 5 = 0.5 F)."""
+    F = res["fwd_flops"]
+    launches = 4 if workload == "c5" else 1          # c5 runs the forward as 4 kernel tiles
+    out = [roof_entry(workload, "fwd_kernel", "mfma", res["fwd_tflops"], peak, "TFLOP/s", res["fwd_ms"] / launches, F / launches)]
+    if "dkdv_ms" in res:
+        out.append(roof_entry(workload, "dkdv_kernel", "mfma", 2.0 * F / res["dkdv_ms"] / 1e9, peak, "TFLOP/s", res["dkdv_ms"], 2.0 * F))
+        out.append(roof_entry(workload, "dq_kernel", "mfma", 0.5 * F / res["dq_ms"] / 1e9, peak, "TFLOP/s", res["dq_ms"], 0.5 * F))
+        nbytes = res["delta_gbps"] * res["delta_ms"] * 1e6
+        out.append(roof_entry(workload, "delta_kernel", "hbm", res["delta_gbps"], HBM_PEAK_GBPS, "GB/s", res["delta_ms"], nbytes))
+    if "merge_ms" in res:
+        out.append(roof_entry(workload, "merge_kernel<4>", "hbm", res["merge_gbps"], HBM_PEAK_GBPS, "GB/s", res["merge_ms"], res["merge_bytes"]))
+    return out
 
 
 def log(*a):
@@ -48,6 +85,7 @@ def probe_lib():
         lib = ctypes.CDLL(path)
         vp, ci = ctypes.c_void_p, ctypes.c_int
         lib.bench_probe_mfma.restype, lib.bench_probe_mfma.argtypes = ci, [vp, vp, ci, ci, vp]
+        lib.bench_probe_mfma_rotating.restype, lib.bench_probe_mfma_rotating.argtypes = ci, [vp, vp, ci, ci, vp]
         lib.bench_stream_mix.restype = ci
         lib.bench_stream_mix.argtypes = [ctypes.POINTER(vp), ci, vp, ctypes.c_int64, ci, ci, vp]
         _probe_lib = lib
@@ -228,7 +266,23 @@ def run_c5(steps, warmup):
     rows = nqb * BLOCK * HEADS
     merge_bytes = (len(tls) + 1) * rows * (128 * 2 + 4)
     m_ms, f_ms = timer.acc["merge"] / steps, timer.acc["fwd_tiles"] / steps
-    return {"workload": "c5", "ms_per_step": wall_ms, "fwd_ms": f_ms, "fwd_tflops": F / f_ms / 1e9, "fwd_flops": F,
+    # the device's rate for the merge's memory pattern without its arithmetic: 4 streams read, 1 written,
+    # 16-byte accesses, one load step per workgroup, on the same buffers
+    import ctypes
+    lib = probe_lib()
+    nb = p_o[0].numel() * 2
+    arr = (ctypes.c_void_p * 4)(*[t.data_ptr() for t in p_o])
+    st = torch.cuda.current_stream().cuda_stream
+    blocks = nb // (256 * 4 * 16)
+    assert lib.bench_stream_mix(arr, 4, o.data_ptr(), nb, blocks, 1, st) == 0
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(10):
+        lib.bench_stream_mix(arr, 4, o.data_ptr(), nb, blocks, 1, st)
+    e1.record()
+    torch.cuda.synchronize()
+    mix_gbps = 5 * nb / (e0.elapsed_time(e1) / 10) / 1e6
+    return {"workload": "c5", "stream_mix_4r1w_gbps": mix_gbps, "merge_frac_of_stream_mix": merge_bytes / m_ms / 1e6 / mix_gbps, "ms_per_step": wall_ms, "fwd_ms": f_ms, "fwd_tflops": F / f_ms / 1e9, "fwd_flops": F,
             "merge_ms": m_ms, "merge_bytes": merge_bytes, "merge_gbps": merge_bytes / m_ms / 1e6,
             "merge_frac_of_hbm": merge_bytes / m_ms / 1e6 / HBM_PEAK_GBPS,
             "fwd_plus_merge_tflops": F / wall_ms / 1e9}
@@ -385,18 +439,24 @@ def probe_mfma(peak):
             "random": torch.randn(512 * 8, dtype=torch.float32, device=dev, generator=g).to(torch.bfloat16)}
     res = {}
     st = torch.cuda.current_stream().cuda_stream
-    for name, t in ops_.items():
-        assert lib.bench_probe_mfma(t.data_ptr(), out.data_ptr(), n_blocks, 2000, st) == 0
+    rot = torch.randn(16 * 256 * 8, dtype=torch.float32, device=dev, generator=g).to(torch.bfloat16)
+    runs = [(name + "_operands_tflops", lib.bench_probe_mfma, t) for name, t in ops_.items()]
+    runs.append(("rotating_random_operands_tflops", lib.bench_probe_mfma_rotating, rot))
+    for key, fn, t in runs:
+        assert fn(t.data_ptr(), out.data_ptr(), n_blocks, 2000, st) == 0
         torch.cuda.synchronize()
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         e0.record()
-        assert lib.bench_probe_mfma(t.data_ptr(), out.data_ptr(), n_blocks, iters, st) == 0
+        assert fn(t.data_ptr(), out.data_ptr(), n_blocks, iters, st) == 0
         e1.record()
         torch.cuda.synchronize()
         ms = e0.elapsed_time(e1)
-        res[name + "_operands_tflops"] = n_blocks * 4 * 4 * iters * 32768.0 / ms / 1e9
-    res["note"] = ("register-only v_mfma_f32_32x32x16_bf16 loop, 2 waves per SIMD; the clock follows power, "
-                   "power follows operand bit activity")
+        res[key] = n_blocks * 4 * 4 * iters * 32768.0 / ms / 1e9
+    res["frac_of_peak_random"] = res["random_operands_tflops"] / peak
+    res["note"] = ("register-only v_mfma_f32_32x32x16_bf16 loops, 2 waves per SIMD: one A/B operand pair reused for ever "
+                   "(constant bits, random N(0,1) bits) and 8x8 random fragments cycled so that the operands change on "
+                   "every instruction; the clock follows power, power follows operand bit activity, so the random "
+                   "figure is the practical ceiling of any bf16 MFMA kernel on this device")
     return res
 
 
@@ -458,26 +518,21 @@ def main():
     else:
         main_res = run_attention(a.workload, a.steps, a.warmup, backward=a.workload in ("c3", "c4"))
     log(json.dumps(main_res))
+    load_traffic()
     backward = "fwd_bwd_tflops" in main_res
     if backward:
         kt = time_bwd_kernels(a.workload, max(3, a.steps // 2))
         F = main_res["fwd_flops"]
-        # dominant kernel: dK/dV.  Algorithmic flops of that launch: 4 of the backward's 5 GEMMs.
-        roof = {"kernel": "dkdv_kernel", "bound": "mfma", "achieved": 2.0 * F / kt["dkdv"] / 1e9, "peak": peak,
-                "unit": "TFLOP/s", "traffic": TRAFFIC_BYTES.get((a.workload, "dkdv_kernel")), "kernel_ms": kt["dkdv"],
-                "algorithmic_flops": 2.0 * F}
         main_res.update(dkdv_ms=kt["dkdv"], dq_ms=kt["dq"], dkdv_tflops=2.0 * F / kt["dkdv"] / 1e9,
                         dq_tflops=0.5 * F / kt["dq"] / 1e9)
         value = main_res["fwd_bwd_tflops"]
         metric = "effective TFLOP/s on active blocks, forward+backward"
     else:
-        launches = 4 if a.workload == "c5" else 1          # c5 runs the forward as 4 kernel tiles
-        roof = {"kernel": "fwd_kernel", "bound": "mfma", "achieved": main_res["fwd_tflops"], "peak": peak,
-                "unit": "TFLOP/s", "traffic": TRAFFIC_BYTES.get((a.workload, "fwd_kernel")),
-                "kernel_ms": main_res["fwd_ms"] / launches, "algorithmic_flops": main_res["fwd_flops"] / launches}
         value = main_res.get("fwd_plus_merge_tflops", main_res["fwd_tflops"])
         metric = "effective TFLOP/s on active blocks, forward"
-    roof["frac"] = roof["achieved"] / roof["peak"]
+    roofs = attention_roofs(a.workload, main_res, peak)
+    # the dominant kernel of the step: dK/dV for the forward+backward workloads, the forward otherwise
+    roof = dict(next(r for r in roofs if r["kernel"] == ("dkdv_kernel" if backward else "fwd_kernel")))
 
     extra = {}
     if not a.no_extra:
@@ -487,6 +542,11 @@ def main():
             torch.cuda.empty_cache()
             r = run_c5(max(3, a.steps // 2), 2) if w == "c5" else \
                 run_attention(w, max(3, a.steps // 2), 2, backward=w in ("c3", "c4"))
+            if "fwd_bwd_tflops" in r:
+                torch.cuda.empty_cache()
+                kt = time_bwd_kernels(w, 3)
+                r.update(dkdv_ms=kt["dkdv"], dq_ms=kt["dq"])
+            roofs += attention_roofs(w, r, peak)
             for key in ("tilelist_sha256", "fwd_flops"):
                 r.pop(key, None)
             r["fwd_frac_of_peak"] = r["fwd_tflops"] / peak
@@ -504,7 +564,7 @@ def main():
                       "seq_q": int(workload_mask(a.workload).shape[0]) * BLOCK,
                       "seq_kv": int(workload_mask(a.workload).shape[1]) * BLOCK},
            "frac_of_bf16_mfma_peak": value / peak, "peak_tflops": peak, "detail": main_res,
-           "fwd_frac_of_peak": main_res["fwd_tflops"] / peak, "roofline": roof, "extra": extra}
+           "fwd_frac_of_peak": main_res["fwd_tflops"] / peak, "roofline": roof, "rooflines": roofs, "extra": extra}
     if not a.no_extra:
         out["mask_builder"] = run_mask_builder(a.workload if a.workload != "c5" else "c3", 20)
         log(json.dumps(out["mask_builder"]))

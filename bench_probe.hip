@@ -35,6 +35,34 @@ __global__ __launch_bounds__(256) void probe_mfma_kernel(const u32x4* in, float*
   out[blockIdx.x * 256 + threadIdx.x] = s;
 }
 
+// Same loop, but every MFMA takes a different pair of operand fragments (8 A x 8 B fragments cycled
+// from registers), as a real GEMM does: the operand latches of the matrix pipe then toggle on every
+// instruction, which the loop above (one A, one B for ever) does not exercise.
+__global__ __launch_bounds__(256) void probe_mfma_rot_kernel(const u32x4* in, float* out, int iters) {
+  bf16x8 a[8], b[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    const u32x4 ra = in[(2 * i) * 256 + threadIdx.x], rb = in[(2 * i + 1) * 256 + threadIdx.x];
+    __builtin_memcpy(&a[i], &ra, 16);
+    __builtin_memcpy(&b[i], &rb, 16);
+  }
+  f32x16 c[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) c[i] = f32x16{0};
+  for (int it = 0; it < iters; it += 8) {
+#pragma unroll
+    for (int u = 0; u < 8; ++u)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) c[i] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[(u + i) & 7], b[(u + 3 * i) & 7], c[i], 0, 0, 0);
+  }
+  float s = 0.f;
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 16; ++j) s += c[i][j];
+  out[blockIdx.x * 256 + threadIdx.x] = s;
+}
+
 constexpr int kMaxSrc = 8;
 struct MixParams {
   const u32x4* src[kMaxSrc];
@@ -85,6 +113,17 @@ extern "C" int bench_probe_mfma(const void* operands, float* out, int n_blocks, 
   if (n_blocks <= 0 || iters <= 0) return -2;
   if (reinterpret_cast<uintptr_t>(operands) & 15) return -4;
   hipLaunchKernelGGL(probe_mfma_kernel, dim3(n_blocks), dim3(256), 0, (hipStream_t)stream,
+                     (const u32x4*)operands, out, iters);
+  return hipGetLastError() == hipSuccess ? 0 : -6;
+}
+
+// operands: 16 x 256 x 16 bytes (8 A and 8 B fragments per thread, interleaved A0 B0 A1 B1 ...);
+// iters is rounded up to a multiple of 8.
+extern "C" int bench_probe_mfma_rotating(const void* operands, float* out, int n_blocks, int iters, void* stream) {
+  if (!operands || !out) return -1;
+  if (n_blocks <= 0 || iters <= 0) return -2;
+  if (reinterpret_cast<uintptr_t>(operands) & 15) return -4;
+  hipLaunchKernelGGL(probe_mfma_rot_kernel, dim3(n_blocks), dim3(256), 0, (hipStream_t)stream,
                      (const u32x4*)operands, out, iters);
   return hipGetLastError() == hipSuccess ? 0 : -6;
 }
