@@ -86,6 +86,7 @@ def probe_lib():
         vp, ci = ctypes.c_void_p, ctypes.c_int
         lib.bench_probe_mfma.restype, lib.bench_probe_mfma.argtypes = ci, [vp, vp, ci, ci, vp]
         lib.bench_probe_mfma_rotating.restype, lib.bench_probe_mfma_rotating.argtypes = ci, [vp, vp, ci, ci, vp]
+        lib.bench_atomic_rate.restype, lib.bench_atomic_rate.argtypes = ci, [vp, ctypes.c_int64, ci, ci, ci, vp]
         lib.bench_stream_mix.restype = ci
         lib.bench_stream_mix.argtypes = [ctypes.POINTER(vp), ci, vp, ctypes.c_int64, ci, ci, vp]
         _probe_lib = lib
@@ -460,6 +461,66 @@ def probe_mfma(peak):
     return res
 
 
+def device_ceilings(peak):
+    """What the device delivers to the simplest possible kernels: register-only MFMA loops with their
+    socket power and clock, L2 atomics and plain stores, streaming reads/writes.  These bound the
+    attention and merge kernels; `python bench.py --device-ceilings` prints them alone."""
+    import ctypes
+    import torch
+    lib = probe_lib()
+    dev = "cuda:0"
+    st = torch.cuda.current_stream().cuda_stream
+    out = {"mfma": probe_mfma(peak)}
+    sampler = PowerSampler()
+    if sampler.exe:
+        sink = torch.empty(512 * 256, dtype=torch.float32, device=dev)
+        g = torch.Generator(device=dev).manual_seed(0)
+        rot = torch.randn(16 * 256 * 8, dtype=torch.float32, device=dev, generator=g).to(torch.bfloat16)
+        one = torch.ones(16 * 256 * 8, dtype=torch.bfloat16, device=dev)
+        for key, fn, t in (("constant", lib.bench_probe_mfma, one), ("random", lib.bench_probe_mfma, rot),
+                           ("rotating_random", lib.bench_probe_mfma_rotating, rot)):
+            out["mfma"][key + "_power"] = sampler.measure(lambda: fn(t.data_ptr(), sink.data_ptr(), 512, 20000, st), 1.5,
+                                                          torch.cuda.synchronize)
+    atom = {}
+    n_blocks, iters = 2048, 2048
+    for mib in (8, 1024):
+        buf = torch.zeros(mib << 18, dtype=torch.float32, device=dev)
+        for mode, name, dwords in ((0, "f32_add", 1), (1, "u32_add", 1), (2, "f64_add", 2), (3, "dword_store", 1)):
+            assert lib.bench_atomic_rate(buf.data_ptr(), buf.numel(), mode, n_blocks, 64, st) == 0
+            torch.cuda.synchronize()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            assert lib.bench_atomic_rate(buf.data_ptr(), buf.numel(), mode, n_blocks, iters, st) == 0
+            e1.record()
+            torch.cuda.synchronize()
+            ops_ = n_blocks * 256 * iters
+            ms = e0.elapsed_time(e1)
+            atom[f"{name}_{mib}MiB"] = {"g_lane_ops_per_s": ops_ / ms / 1e6, "payload_gbps": ops_ * 4 * dwords / ms / 1e6}
+        del buf
+    out["l2_atomics"] = atom
+    out["l2_atomics_note"] = ("2048 workgroups x 256 threads x 2048 operations, a wave instruction covers two 128-byte lines; "
+                              "target region 8 MiB (stays in L2) and 1 GiB")
+    n = 512 << 20
+    srcs = [torch.empty(n, dtype=torch.uint8, device=dev) for _ in range(4)]
+    dst = torch.empty(n, dtype=torch.uint8, device=dev)
+    mix = {}
+    for ns in (1, 2, 4):
+        arr = (ctypes.c_void_p * ns)(*[t.data_ptr() for t in srcs[:ns]])
+        blocks = n // (256 * 4 * 16)
+        lib.bench_stream_mix(arr, ns, dst.data_ptr(), n, blocks, 1, st)
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(10):
+            lib.bench_stream_mix(arr, ns, dst.data_ptr(), n, blocks, 1, st)
+        e1.record()
+        torch.cuda.synchronize()
+        mix[f"{ns}_read_1_write_gbps"] = (ns + 1) * n / (e0.elapsed_time(e1) / 10) / 1e6
+    out["stream_mix"] = mix
+    out["stream_mix_note"] = "512 MiB per stream, 16-byte non-temporal accesses, one load step per workgroup"
+    return out
+
+
 def cpu_baseline():
     """The reference's block-loop path restated on the CPU (oracle.block_loop_fwd), timed on
     config 1 exactly: B=1, S=8192, Nh=8, d=128, fp32, 16x16 causal block grid, forward only."""
@@ -493,6 +554,8 @@ def main():
     ap.add_argument("--workload", default="c3", choices=["c2", "c3", "c4", "c5"])
     ap.add_argument("--no-extra", action="store_true", help="skip the other workloads")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    ap.add_argument("--device-ceilings", action="store_true",
+                    help="print only the device's ceilings (MFMA loops, L2 atomics, streaming mixes) as one JSON line")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one plain 1 GiB device copy (known size, for scaling rocprof byte counters)")
     a = ap.parse_args()
@@ -507,6 +570,9 @@ def main():
     peak = prop.multi_processor_count * FLOP_PER_CLK_PER_CU * clock_ghz / 1e3      # TFLOP/s
     log(f"device {prop.name}: {prop.multi_processor_count} CUs @ {clock_ghz:.2f} GHz -> bf16 MFMA peak {peak:.1f} TFLOP/s")
 
+    if a.device_ceilings:
+        print(json.dumps(device_ceilings(peak)), flush=True)
+        return
     if a.calibrate_copy:
         src = torch.empty(1 << 30, dtype=torch.uint8, device="cuda:0")
         dst = torch.empty_like(src)

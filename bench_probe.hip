@@ -8,6 +8,10 @@
 //                      of any bf16 MFMA kernel fed with ordinary data.
 //   bench_stream_mix   n_src streams read and one written with 16-byte accesses, the access
 //                      shape of the merge kernel: the device's rate for that read:write mix.
+//   bench_atomic_rate  device-wide rate of L2 atomics (fp32 add, u32 add, f64 add) and of plain dword
+//                      stores with the access shape a backward that sums dQ with atomics would have
+//                      (a wave instruction covers two 128-byte lines): the figure that decides
+//                      between recomputing S and dP in a second kernel and one fused kernel.
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
@@ -61,6 +65,19 @@ __global__ __launch_bounds__(256) void probe_mfma_rot_kernel(const u32x4* in, fl
 #pragma unroll
     for (int j = 0; j < 16; ++j) s += c[i][j];
   out[blockIdx.x * 256 + threadIdx.x] = s;
+}
+
+template <int MODE>
+__global__ __launch_bounds__(256) void atomic_rate_kernel(void* buf, int64_t n_dwords, int iters) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int64_t base = ((int64_t)blockIdx.x * 4 + wave) * 64 * 64;      // each wave walks its own region
+  for (int it = 0; it < iters; ++it) {
+    const int64_t off = (base + (int64_t)it * 64 + lane) % n_dwords;
+    if (MODE == 0) __builtin_amdgcn_global_atomic_fadd_f32((__attribute__((address_space(1))) float*)buf + off, 1.0f);
+    if (MODE == 1) atomicAdd((unsigned*)buf + off, 1u);
+    if (MODE == 2) atomicAdd((double*)buf + (off >> 1), 1.0);
+    if (MODE == 3) ((volatile unsigned*)buf)[off] = 1u;
+  }
 }
 
 constexpr int kMaxSrc = 8;
@@ -152,4 +169,19 @@ extern "C" int bench_stream_mix(const void* const* srcs, int n_src, void* dst, i
     case 7: return launch_mix<7>(p, n_blocks, non_temporal, st);
     default: return launch_mix<8>(p, n_blocks, non_temporal, st);
   }
+}
+
+// mode: 0 fp32 atomic add (no return), 1 u32 atomic add, 2 f64 atomic add, 3 plain dword store.
+// n_blocks x 256 threads, each issuing `iters` operations on buf[0 .. n_dwords) (device, 8-byte aligned).
+extern "C" int bench_atomic_rate(void* buf, int64_t n_dwords, int mode, int n_blocks, int iters, void* stream) {
+  if (!buf) return -1;
+  if (n_dwords < 4096 || n_dwords % 2 || n_blocks <= 0 || iters <= 0 || mode < 0 || mode > 3) return -2;
+  hipStream_t st = (hipStream_t)stream;
+  switch (mode) {
+    case 0: hipLaunchKernelGGL(atomic_rate_kernel<0>, dim3(n_blocks), dim3(256), 0, st, buf, n_dwords, iters); break;
+    case 1: hipLaunchKernelGGL(atomic_rate_kernel<1>, dim3(n_blocks), dim3(256), 0, st, buf, n_dwords, iters); break;
+    case 2: hipLaunchKernelGGL(atomic_rate_kernel<2>, dim3(n_blocks), dim3(256), 0, st, buf, n_dwords, iters); break;
+    default: hipLaunchKernelGGL(atomic_rate_kernel<3>, dim3(n_blocks), dim3(256), 0, st, buf, n_dwords, iters); break;
+  }
+  return hipGetLastError() == hipSuccess ? 0 : -6;
 }
