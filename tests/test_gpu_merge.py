@@ -157,3 +157,32 @@ def test_update_out_and_lse_bf16_in_place_and_statistics_layouts():
         ops.update_out_and_lse(None, None, outs[0].to(DEV), lses[0].to(DEV), slice_=(slice(None),))
     with pytest.raises(ValueError):
         ops.update_out_and_lse(run_o, run_l, outs[1][:, :32].to(DEV), blk_l)
+
+
+@pytest.mark.parametrize("run_dtype,blk_dtype", [(torch.float32, torch.bfloat16), (torch.bfloat16, torch.float32),
+                                                 (torch.float32, torch.float32)])
+def test_update_out_and_lse_views_dtypes_and_layouts(run_dtype, blk_dtype):
+    """Strided targets (a head range and a row range of a larger running tensor, batch 2), rows in
+    bf16 or fp32 on either side, and the running statistics kept in the kernels' [B,Nh,S] layout:
+    one ua_merge_update call each, against the stabilised oracle."""
+    B, S, Nh = 2, 53, 6
+    g = torch.Generator().manual_seed(17)
+    run_o = torch.randn(B, S, Nh, 128, generator=g).to(run_dtype)
+    blk_o = torch.randn(B, 20, 4, 128, generator=g).to(blk_dtype)
+    run_l = torch.randn(B, Nh, S, generator=g) * 2.0
+    blk_l = torch.randn(B, 4, 20, generator=g) * 2.0
+    sl_rows, sl_heads = slice(30, 50), slice(1, 5)
+    ro, rl = ao.merge_partials([run_o[:, sl_rows, sl_heads], blk_o], [run_l[:, sl_heads, sl_rows], blk_l])
+    d_o, d_l = run_o.to(DEV), run_l.to(DEV)
+    keep_o, keep_l = d_o.clone(), d_l.clone()
+    tgt_o = d_o[:, sl_rows, sl_heads]                      # strided view: written in place through slice_
+    tgt_l = d_l[:, sl_heads, sl_rows]
+    o, l = ops.update_out_and_lse(tgt_o, tgt_l, blk_o.to(DEV), blk_l.to(DEV), slice_=(slice(None),))
+    torch.cuda.synchronize()
+    tol = ATOL_O if run_dtype == torch.bfloat16 else (1e-2 if blk_dtype == torch.bfloat16 else 3e-5)
+    assert max_abs(d_o[:, sl_rows, sl_heads], ro.to(run_dtype).float()) <= tol
+    assert lse_rel_err(d_l[:, sl_heads, sl_rows], rl) <= 1e-5
+    # everything outside the target is untouched
+    mask_o = torch.ones_like(d_o, dtype=torch.bool); mask_o[:, sl_rows, sl_heads] = False
+    mask_l = torch.ones_like(d_l, dtype=torch.bool); mask_l[:, sl_heads, sl_rows] = False
+    assert torch.equal(d_o[mask_o], keep_o[mask_o]) and torch.equal(d_l[mask_l], keep_l[mask_l])

@@ -33,6 +33,27 @@ def test_device_builder_bit_exact(make, block):
         assert np.array_equal(got, getattr(host, f)), f
 
 
+def test_device_builder_reports_invalid_mask_entries():
+    """The host builder rejects a mask value other than 0/1/2 (UA_ERR_MASK); the device builder cannot
+    return an error without a synchronisation, treats the entry as EMPTY and counts it."""
+    m = masks.config_strided(8, 2, 4).copy()
+    ok = build_tile_list_device(torch.from_numpy(m).to(DEV), 256, check=True)
+    bad = m.copy()
+    bad[3, 1] = 7
+    with pytest.raises(RuntimeError, match="EMPTY"):
+        build_tile_list(bad, 256)
+    with pytest.raises(ValueError, match="1 entries"):
+        build_tile_list_device(torch.from_numpy(bad).to(DEV), 256, check=True)
+    as_empty = bad.copy()
+    as_empty[3, 1] = 0
+    want = build_tile_list(as_empty, 256)
+    got = build_tile_list_device(torch.from_numpy(bad).to(DEV), 256, nnz=want.nnz)
+    torch.cuda.synchronize()
+    for f in FIELDS:
+        assert np.array_equal(got[f].cpu().numpy(), getattr(want, f)), f
+    assert ok["row_ptr"].shape[0] == 8 * 2 + 1
+
+
 @pytest.mark.parametrize("causal", [False, True])
 @pytest.mark.parametrize("sq,sk", [(256, 256), (128, 384), (384, 384), (384, 128)])
 def test_flash_attn_shim(causal, sq, sk):
