@@ -159,8 +159,9 @@ int ua_merge(const void *const *o_parts, const float *const *lse_parts, int n_pa
  * pointer offset), statistics fp32 in either the reference's running layout [B, S, Nh, 1]
  * (strides S*Nh, Nh, 1) or the kernels' [B, Nh, S] (strides Nh*S, 1, S).  `*_is_fp32` select
  * fp32 or bf16 rows (the reference's running `out` turns fp32 after its first update).
- * new_out / new_lse may alias out / lse (the slice_ path) or be separate buffers.  Row strides
- * must keep rows 16-byte aligned.                                                          */
+ * new_out / new_lse may be exactly out / lse (the slice_ path: same pointer, same strides) or
+ * buffers that do not overlap them; partial overlap is undefined.  Row strides must keep rows
+ * 16-byte aligned (multiples of 8 bf16 / 4 fp32 elements).                                   */
 int ua_merge_update(const void *out, const float *lse, const void *block_out, const float *block_lse,
                     void *new_out, float *new_lse, int batch, int n_rows, int n_heads, int head_dim,
                     int out_is_fp32, int block_is_fp32, int new_is_fp32,
