@@ -12,7 +12,7 @@ namespace ua {
 
 constexpr int kCopyThreads = 256;
 constexpr int kCopyVecs = 4;                                   // 16-byte vectors per thread and step
-constexpr int kTargetGroups = 4096;                            // workgroups per launch, 16 per CU
+constexpr int kTargetGroups = 32768;                           // workgroups per launch, 128 per CU
 constexpr int64_t kSegBytes = (int64_t)kCopyThreads * kCopyVecs * 16;   // per workgroup and step
 
 struct PermuteParams {
@@ -30,8 +30,8 @@ __global__ __launch_bounds__(kCopyThreads) void permute_chunks_kernel(PermutePar
   const int64_t fused = id, split = ((int64_t)y * 2 + c) * p.n_b + b;
   const unsigned char* s = p.src + (p.gather ? split : fused) * p.chunk_bytes;
   unsigned char* d = p.dst + (p.gather ? fused : split) * p.chunk_bytes;
-  // a workgroup walks its chunk in strides of the grid's width: few, long-lived workgroups keep
-  // more loads in flight than one short workgroup per segment
+  // a workgroup walks its chunk in strides of the grid's width.  Measured on a 4 GiB buffer:
+  // 4096 workgroups 5.57 TB/s, 32768 5.98 TB/s, one per segment 5.86 TB/s
   for (int64_t seg0 = (int64_t)blockIdx.x * kSegBytes; seg0 < p.chunk_bytes; seg0 += (int64_t)gridDim.x * kSegBytes) {
     u32x4 v[kCopyVecs];
 #pragma unroll
