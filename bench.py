@@ -89,6 +89,7 @@ def probe_lib():
         lib.bench_atomic_rate.restype, lib.bench_atomic_rate.argtypes = ci, [vp, ctypes.c_int64, ci, ci, ci, vp]
         lib.bench_stream_mix.restype = ci
         lib.bench_stream_mix.argtypes = [ctypes.POINTER(vp), ci, vp, ctypes.c_int64, ci, ci, vp]
+        lib.bench_issue_mix.restype, lib.bench_issue_mix.argtypes = ci, [vp, ci, ci, ci, ci, vp]
         _probe_lib = lib
     return _probe_lib
 
@@ -518,6 +519,32 @@ def device_ceilings(peak):
         mix[f"{ns}_read_1_write_gbps"] = (ns + 1) * n / (e0.elapsed_time(e1) / 10) / 1e6
     out["stream_mix"] = mix
     out["stream_mix_note"] = "512 MiB per stream, 16-byte non-temporal accesses, one load step per workgroup"
+    del srcs, dst
+    # instruction mix of the forward per 32 keys, registers and LDS only, zero data: what share of the time the bare
+    # 16-MFMA loop takes
+    sink = torch.empty(256 * 512, dtype=torch.float32, device=dev)
+    names = ("16 MFMA", "16 MFMA + 40 fma + 16 exp2", "16 MFMA + 8 ds_read_b128 + 16 ds_read_b64_tr_b16",
+             "16 MFMA + 40 fma + 16 exp2 + 8 ds_read_b128 + 16 ds_read_b64_tr_b16", "40 fma + 16 exp2", "8 ds_read_b128 + 16 ds_read_b64_tr_b16")
+    issue = {}
+    for wps in (1, 2):
+        ms = []
+        for mix in range(6):
+            assert lib.bench_issue_mix(sink.data_ptr(), 256, wps, mix, 2000, st) == 0
+            torch.cuda.synchronize()
+            best = float("inf")
+            for _ in range(3):
+                e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                e0.record()
+                assert lib.bench_issue_mix(sink.data_ptr(), 256, wps, mix, 20000, st) == 0
+                e1.record()
+                torch.cuda.synchronize()
+                best = min(best, e0.elapsed_time(e1))
+            ms.append(best)
+        issue[f"{wps}_waves_per_simd"] = {n: {"ms": t, "rel_to_bare_mfma_loop": t / ms[0], "matrix_pipe_share": ms[0] / t if i < 4 else None}
+                                           for i, (n, t) in enumerate(zip(names, ms))}
+    out["issue_mix"] = issue
+    out["issue_mix_note"] = ("256 workgroups (one per CU), 20000 iterations per wave, zero operands (the clock stays at its maximum); "
+                             "matrix_pipe_share = time of the bare MFMA loop / time of the mix")
     return out
 
 

@@ -12,6 +12,11 @@
 //                      stores with the access shape a backward that sums dQ with atomics would have
 //                      (a wave instruction covers two 128-byte lines): the figure that decides
 //                      between recomputing S and dP in a second kernel and one fused kernel.
+//   bench_issue_mix    one loop iteration = 16 MFMAs plus the vector and LDS instructions that the forward kernel
+//                      issues per 32 keys (40 fma-class, 16 exp2, 8 ds_read_b128, 16 ds_read_b64_tr_b16), on zero
+//                      data, registers and LDS only, 1 or 2 waves per SIMD: time of the bare MFMA loop / time of a
+//                      mix = the matrix-pipe occupancy that this instruction mix allows before barriers, copies
+//                      and power come in.
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
@@ -78,6 +83,60 @@ __global__ __launch_bounds__(256) void atomic_rate_kernel(void* buf, int64_t n_d
     if (MODE == 2) atomicAdd((double*)buf + (off >> 1), 1.0);
     if (MODE == 3) ((volatile unsigned*)buf)[off] = 1u;
   }
+}
+
+typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4;
+// M MFMAs per iteration; per MFMA slot V/M fma, X/M exp2 interleaved behind it; L 128-bit and T transposing
+// 64-bit LDS reads issued at the top of the iteration and consumed at its end.
+template <int M, int V, int X, int L, int T>
+__global__ __launch_bounds__(512) void issue_mix_kernel(float* out, int iters, float kk) {
+  __shared__ __attribute__((aligned(1024))) unsigned char lds[32768];
+  typedef __attribute__((address_space(3))) bf16x4 lds_bf16x4;
+  for (int i = threadIdx.x; i < 8192; i += blockDim.x) reinterpret_cast<uint32_t*>(lds)[i] = 0;
+  __syncthreads();
+  f32x16 c[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) c[i] = f32x16{0};
+  const bf16x8 a = {0}, b = {0};
+  float r[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) r[i] = kk * threadIdx.x;
+  const int lane = threadIdx.x & 63;
+  constexpr int N = M > 0 ? M : 16;
+  constexpr int VS = (V + N - 1) / N, XS = (X + N - 1) / N;
+  for (int it = 0; it < iters; ++it) {
+    u32x4 lv[L > 0 ? L : 1];
+    bf16x4 tv[T > 0 ? T : 1];
+#pragma unroll
+    for (int j = 0; j < L; ++j) lv[j] = *reinterpret_cast<const u32x4*>(lds + lane * 16 + (j & 15) * 1024);
+#pragma unroll
+    for (int j = 0; j < T; ++j) tv[j] = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((lds_bf16x4*)(lds + lane * 8 + (j & 31) * 512));
+    if (L + T > 0) __builtin_amdgcn_sched_group_barrier(0x100, L + T, 0);
+#pragma unroll
+    for (int i = 0; i < N; ++i) {
+      if (M > 0) c[i & 3] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c[i & 3], 0, 0, 0);
+#pragma unroll
+      for (int j = 0; j < VS; ++j) if (i * VS + j < V) r[(i + j) & 7] = __builtin_fmaf(r[(i + j) & 7], kk, kk);
+#pragma unroll
+      for (int j = 0; j < XS; ++j) if (i * XS + j < X) r[(i + j + 4) & 7] = __builtin_amdgcn_exp2f(r[(i + j + 4) & 7]);
+      if (M > 0) __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      if (V + X > 0) __builtin_amdgcn_sched_group_barrier(0x002, VS + XS, 0);
+    }
+    uint32_t acc = 0;
+#pragma unroll
+    for (int j = 0; j < L; ++j) acc ^= lv[j][0] ^ lv[j][3];
+#pragma unroll
+    for (int j = 0; j < T; ++j) acc ^= __builtin_bit_cast(uint32_t, __builtin_shufflevector(tv[j], tv[j], 0, 1));
+    if (L + T > 0) r[0] += __builtin_bit_cast(float, acc);
+  }
+  float s = 0.f;
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 16; ++j) s += c[i][j];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) s += r[i];
+  out[blockIdx.x * blockDim.x + threadIdx.x] = s;
 }
 
 constexpr int kMaxSrc = 8;
@@ -182,6 +241,25 @@ extern "C" int bench_atomic_rate(void* buf, int64_t n_dwords, int mode, int n_bl
     case 1: hipLaunchKernelGGL(atomic_rate_kernel<1>, dim3(n_blocks), dim3(256), 0, st, buf, n_dwords, iters); break;
     case 2: hipLaunchKernelGGL(atomic_rate_kernel<2>, dim3(n_blocks), dim3(256), 0, st, buf, n_dwords, iters); break;
     default: hipLaunchKernelGGL(atomic_rate_kernel<3>, dim3(n_blocks), dim3(256), 0, st, buf, n_dwords, iters); break;
+  }
+  return hipGetLastError() == hipSuccess ? 0 : -6;
+}
+
+// mix: 0 = 16 MFMA; 1 = + 40 fma + 16 exp2; 2 = 16 MFMA + 8 ds_read_b128 + 16 ds_read_b64_tr_b16; 3 = all of them;
+// 4 = the vector work alone; 5 = the LDS reads alone.  waves_per_simd 1 or 2 (256 or 512 threads per workgroup, one
+// workgroup per CU when n_blocks = number of CUs).  out: n_blocks x 512 floats.
+extern "C" int bench_issue_mix(float* out, int n_blocks, int waves_per_simd, int mix, int iters, void* stream) {
+  if (!out) return -1;
+  if (n_blocks <= 0 || iters <= 0 || (waves_per_simd != 1 && waves_per_simd != 2) || mix < 0 || mix > 5) return -2;
+  const dim3 g(n_blocks), t(256 * waves_per_simd);
+  hipStream_t st = (hipStream_t)stream;
+  switch (mix) {
+    case 0: hipLaunchKernelGGL((issue_mix_kernel<16, 0, 0, 0, 0>), g, t, 0, st, out, iters, 0.f); break;
+    case 1: hipLaunchKernelGGL((issue_mix_kernel<16, 40, 16, 0, 0>), g, t, 0, st, out, iters, 0.f); break;
+    case 2: hipLaunchKernelGGL((issue_mix_kernel<16, 0, 0, 8, 16>), g, t, 0, st, out, iters, 0.f); break;
+    case 3: hipLaunchKernelGGL((issue_mix_kernel<16, 40, 16, 8, 16>), g, t, 0, st, out, iters, 0.f); break;
+    case 4: hipLaunchKernelGGL((issue_mix_kernel<0, 40, 16, 0, 0>), g, t, 0, st, out, iters, 0.f); break;
+    default: hipLaunchKernelGGL((issue_mix_kernel<0, 0, 0, 8, 16>), g, t, 0, st, out, iters, 0.f); break;
   }
   return hipGetLastError() == hipSuccess ? 0 : -6;
 }
