@@ -67,7 +67,27 @@ def test_argument_checks_without_gpu(lib):
                              s, s, s, s, s, 0.1, None) == -1
     assert lib.ua_bsa_bwd_dkdv(buf, buf, buf, buf, buf, buf, buf, buf, buf, buf, None, buf, 1, 1, 1, 1, 1, 128,
                                s, s, s, s, s, s, 0.1, None) == -1
-    for code in range(-7, 1):
+    # in-place update of a running (out, lse): NULL, head_dim, sizes, row alignment (fp32 rows: strides in multiples of 4)
+    ls = (ctypes.c_int64 * 3)(16, 1, 16)
+    ok = (buf, buf, buf, buf, buf, buf)
+    assert lib.ua_merge_update(*ok[:5], None, 1, 16, 1, 128, 0, 0, 0, s, ls, s, ls, s, ls, None) == -1
+    assert lib.ua_merge_update(*ok, 1, 16, 1, 64, 0, 0, 0, s, ls, s, ls, s, ls, None) == -3
+    assert lib.ua_merge_update(*ok, 1, 0, 1, 128, 0, 0, 0, s, ls, s, ls, s, ls, None) == -2
+    odd = (ctypes.c_int64 * 3)(128 * 128, 132, 128)          # bf16 rows need strides in multiples of 8
+    assert lib.ua_merge_update(*ok, 1, 16, 1, 128, 0, 0, 0, odd, ls, s, ls, s, ls, None) == -4
+    # device tile-list builders: NULL, sizes, and the no-allocation variant's limit on the number of lines
+    args = (buf,) * 8
+    assert lib.ua_tilelist_build_device(buf, 1, 1, 4, *args, None, None) == -1
+    assert lib.ua_tilelist_build_device(buf, 0, 1, 4, *args, buf, None) == -2
+    assert lib.ua_tilelist_build_device_noalloc(None, 1, 1, 4, *args, None, None) == -1
+    assert lib.ua_tilelist_build_device_noalloc(buf, 16384, 16384, 4, *args, None, None) == -8
+    assert lib.ua_tilelist_build_device_noalloc(buf, 8192, 8192, 4, *args, None, None) == -8    # 65536 lines > 65532
+    # column-buffer layout changes: NULL, sizes, alignment, overlap
+    assert lib.ua_cols_gather(None, buf, 2, 1, 1024, None) == -1
+    assert lib.ua_cols_gather(buf, buf + (1 << 20), 0, 1, 1024, None) == -2
+    assert lib.ua_cols_scatter(buf, buf + (1 << 20), 2, 1, 1020, None) == -4
+    assert lib.ua_cols_scatter(buf, buf + 16, 2, 1, 1024, None) == -2                            # overlapping buffers
+    for code in range(-8, 1):
         assert lib.ua_strerror(code) != b"unknown error code"
     assert lib.ua_strerror(-99) == b"unknown error code"
 

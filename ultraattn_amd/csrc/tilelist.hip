@@ -283,7 +283,7 @@ static int check_device_builder_args(const uint8_t* block_mask, int n_qblocks, i
     return UA_ERR_NULL;
   if (n_qblocks <= 0 || n_kblocks <= 0 || rate <= 0) return UA_ERR_SHAPE;
   if ((int64_t)n_qblocks * rate > (1 << 24) || (int64_t)n_kblocks * rate > (1 << 24)) return UA_ERR_SHAPE;
-  return check_device();
+  return UA_OK;
 }
 
 }  // namespace ua
@@ -296,6 +296,7 @@ extern "C" int ua_tilelist_build_device(const uint8_t* block_mask, int n_qblocks
   if (!work) return UA_ERR_NULL;
   if (int rc = check_device_builder_args(block_mask, n_qblocks, n_kblocks, rate, row_ptr, col_idx, flag, col_ptr,
                                          row_idx, cflag, q_order, k_order)) return rc;
+  if (int rc = check_device()) return rc;
   const int nqt = n_qblocks * rate, nkt = n_kblocks * rate;
   return build_device_impl(block_mask, n_qblocks, n_kblocks, rate, row_ptr, col_idx, flag, col_ptr, row_idx, cflag,
                            q_order, k_order, work, work + nqt + nkt + 2, (hipStream_t)stream);
@@ -327,6 +328,7 @@ extern "C" int ua_tilelist_build_device_noalloc(const uint8_t* block_mask, int n
                                          row_idx, cflag, q_order, k_order)) return rc;
   const int64_t lines = (int64_t)n_qblocks * rate + (int64_t)n_kblocks * rate;
   if (lines > UA_NOALLOC_MAX_LINES) return UA_ERR_TOO_LARGE;
+  if (int rc = check_device()) return rc;
   int32_t* work = nullptr;
   if (int rc = scratch_of_current_device(&work)) return rc;
   // the counts are written before they are read and the invalid-entry count is stored, not
