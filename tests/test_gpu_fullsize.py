@@ -46,14 +46,16 @@ def test_config1_exact_workload_vs_cpu_block_loop():
     assert max_abs(dq, rq) <= ATOL_O and max_abs(dk, rk) <= ATOL_O and max_abs(dv, rv) <= ATOL_O
 
 
-@pytest.mark.parametrize("cfg,head", [("c3", 5), ("c4", 26)])
+@pytest.mark.parametrize("cfg,head", [("c2", 17), ("c3", 5), ("c4", 26), ("c5", 9)])
 def test_whole_head_at_full_size(cfg, head):
-    """Configurations 3 and 4 at their real shape (S=131072, Nh=32): every row of one head."""
-    mask = {"c3": masks.config_strided(), "c4": masks.config_global_local()}[cfg]
+    """Configurations 2 to 5 at their real shape (Nh=32; S=32768, 131072, 131072 and the streaming
+    shard's 65536 query rows against 524288 keys): every row of one head, forward and backward."""
+    mask = {"c2": masks.config_causal(64), "c3": masks.config_strided(), "c4": masks.config_global_local(),
+            "c5": masks.config_streaming_shard()}[cfg]
     block, nh = 512, 32
     g = torch.Generator(device=DEV).manual_seed(0)
     mk = lambda n: torch.randn(1, n * block, nh, 128, device=DEV, dtype=torch.float32, generator=g).to(torch.bfloat16)
-    q, k, v, do = mk(256), mk(256), mk(256), mk(256)
+    q, k, v, do = mk(mask.shape[0]), mk(mask.shape[1]), mk(mask.shape[1]), mk(mask.shape[0])
     tl = build_tile_list(mask, block)
     o, lse = ops.bsa_fwd(q, k, v, tl, SCALE)
     dq, dk, dv = ops.bsa_bwd(do, q, k, v, o, lse, tl, SCALE)
