@@ -75,7 +75,7 @@ int ua_tilelist_build(const uint8_t *block_mask, int n_qblocks, int n_kblocks, i
 
 /* Device-side variant: `block_mask` and all outputs are DEVICE arrays (sizes as above, from
  * ua_tilelist_size on a host copy or an upper bound nnz <= n_qtiles*n_ktiles); `work` is a
- * device scratch of (n_qtiles + n_ktiles + 3) int32.  Produces the same arrays bit for bit.
+ * device scratch of (n_qtiles + n_ktiles + 7) int32.  Produces the same arrays bit for bit.
  * The mask cannot be validated without a synchronisation: an entry that is not 0, 1 or 2 is
  * treated as EMPTY, and work[n_qtiles + n_ktiles + 2] receives the number of such entries (0 for
  * a valid mask; the host builder returns UA_ERR_MASK instead) for the caller to read later.  */
@@ -87,7 +87,7 @@ int ua_tilelist_build_device(const uint8_t *block_mask, int n_qblocks, int n_kbl
 /* No counterpart in the reference.  For callers that cannot allocate device memory (code under
  * HIP graph capture, tight serving loops, harnesses that forbid it): the same builder as
  * ua_tilelist_build_device with the `work` scratch taken from a fixed array inside the library
- * (256 KiB per GPU, held until the process ends) instead of from the caller.  Limit:
+ * (256 KiB + 32 B per GPU, held until the process ends) instead of from the caller.  Limit:
  * n_qtiles + n_ktiles <= UA_NOALLOC_MAX_LINES, else UA_ERR_TOO_LARGE.  `n_invalid` (device,
  * may be NULL) receives the number of mask entries that are not 0, 1 or 2.  It calls no
  * hipMalloc/hipFree.  All calls on one GPU share the array: calls that overlap in time on the

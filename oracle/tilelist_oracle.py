@@ -124,27 +124,39 @@ def build_tile_list(block_table: np.ndarray, rate: int) -> Dict[str, np.ndarray]
     for _, l, _ in by_col:
         col_ptr[l + 1] += 1
     col_ptr = np.cumsum(col_ptr, dtype=np.int64).astype(np.int32)
-    q_order = launch_order(row_ptr, col_idx)
-    k_order = launch_order(col_ptr, row_idx)
+    q_order = launch_order(row_ptr, col_idx, rate, rate - 1)
+    k_order = launch_order(col_ptr, row_idx, rate, 0)
     return dict(row_ptr=row_ptr, col_idx=col_idx, flag=flag, col_ptr=col_ptr, row_idx=row_idx,
                 cflag=cflag, q_order=q_order, k_order=k_order, n_qtiles=nqt, n_ktiles=nkt)
 
 
-def launch_order(ptr: np.ndarray, idx: np.ndarray) -> np.ndarray:
-    """Launch order of the rows of a CSR (or columns of a CSC).  Rows much longer than average
-    (length * n_rows > 2 * nnz) come first, longest first, so that they cannot end up as the
-    tail of the launch; all other rows follow in lexicographic order of their index lists
-    (a list that is a prefix of another sorts after it), which puts rows that walk the same
-    K/V tiles next to each other.  Ties by row number."""
+def launch_order(ptr: np.ndarray, idx: np.ndarray, rate: int, longest_sub: int) -> np.ndarray:
+    """Launch order of the rows of a CSR (``longest_sub = rate - 1``) or the columns of a CSC
+    (``longest_sub = 0``).  Rows much longer than average (length * n_rows > 2 * nnz) come first,
+    longest first, so that they cannot end up as the tail of the launch.  The others are ordered by
+    their anchor index: the first index of the list, or the last one if the last indices take
+    fewer distinct values than the first ones over these rows (the lists are then read backwards
+    below); then by the length of their block line, longest first (measured as the list length of
+    the block's longest tile, sub-tile ``longest_sub``); then lexicographically by the rest of
+    their index lists (a list that is a prefix of another sorts after it); ties by row number.
+    Rows without tiles come last."""
     n = len(ptr) - 1
     nnz = int(ptr[-1])
     inf = 1 << 40
+    lists = [tuple(int(x) for x in idx[ptr[i]:ptr[i + 1]]) for i in range(n)]
+    ruled = [l for l in lists if l and not len(l) * n > 2 * nnz]
+    from_end = len({l[-1] for l in ruled}) < len({l[0] for l in ruled})
 
     def key(i):
-        lst = tuple(int(x) for x in idx[ptr[i]:ptr[i + 1]])
+        lst = lists[i]
         if len(lst) * n > 2 * nnz:
             return (0, (-len(lst),), i)
-        return (1, lst + (inf,), i)
+        if not lst:
+            return (2, (), i)
+        ref = i // rate * rate + longest_sub
+        if from_end:
+            lst = lst[::-1]
+        return (1, (lst[0], -int(ptr[ref + 1] - ptr[ref])) + lst[1:] + (inf,), i)
     return np.array(sorted(range(n), key=key), dtype=np.int32).reshape(-1)
 
 

@@ -63,16 +63,36 @@ def test_full_size_digests(golden_dir, lib):
 
 
 def test_launch_order_groups_rows_with_common_tiles(lib):
-    """Independent statement of the order: plain Python sort of the padded index lists."""
+    """Independent statement of the order: plain Python sort of (first tile, -length of the block
+    row, rest of the list padded so that a prefix sorts last, row)."""
     m = masks.config_strided(32)
-    tl = build_tile_list(m, block=256)
+    rate = 2
+    tl = build_tile_list(m, block=128 * rate)
     lists = [tuple(tl.col_idx[tl.row_ptr[r]:tl.row_ptr[r + 1]]) for r in range(tl.n_qtiles)]
-    assert not any(len(l) * tl.n_qtiles > 2 * tl.nnz for l in lists)
-    want = sorted(range(tl.n_qtiles), key=lambda r: (lists[r] + (10 ** 9,), r))
-    assert tl.q_order.tolist() == want
+    assert not any(len(l) * tl.n_qtiles > 2 * tl.nnz for l in lists) and all(lists)
+    block_len = lambda r: len(lists[r // rate * rate + rate - 1])
+    want = sorted(range(tl.n_qtiles), key=lambda r: ((lists[r][0], -block_len(r)) + lists[r][1:] + (10 ** 9,), r))
+    order = tl.q_order.tolist()
+    assert order == want
     # the two query tiles of one strided block sit next to each other
-    pos = {r: i for i, r in enumerate(tl.q_order.tolist())}
+    pos = {r: i for i, r in enumerate(order)}
     assert all(abs(pos[2 * b] - pos[2 * b + 1]) == 1 for b in range(32))
+    # rows that start on the same tile: the longer block rows come first
+    for a, b in zip(order[:-1], order[1:]):
+        if lists[a][0] == lists[b][0]:
+            assert block_len(a) >= block_len(b)
+    # the key side of the same mask: every column starts at its own diagonal tile, while the columns of
+    # one residue class end on the same query tiles, so the order is anchored at the END of the lists
+    cols = [tuple(tl.row_idx[tl.col_ptr[c]:tl.col_ptr[c + 1]]) for c in range(tl.n_ktiles)]
+    assert len({c[-1] for c in cols}) < len({c[0] for c in cols})
+    col_len = lambda c: len(cols[c // rate * rate])
+    want_k = sorted(range(tl.n_ktiles), key=lambda c: ((cols[c][-1], -col_len(c)) + cols[c][-2::-1] + (10 ** 9,), c))
+    assert tl.k_order.tolist() == want_k
+    ends = [cols[c][-1] for c in tl.k_order.tolist()]
+    assert ends == sorted(ends)
+    # a plain causal mask: all columns end on the last query tile; the longest column (0) comes first
+    tc = build_tile_list(masks.config_causal(8), block=256)
+    assert tc.k_order.tolist() == list(range(tc.n_ktiles))
     # global rows of the global+local mask are the long ones and come first
     tg = build_tile_list(masks.config_global_local(64, 2, 4), block=128)
     assert sorted(tg.q_order[:2].tolist()) == [0, 1]

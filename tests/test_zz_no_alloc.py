@@ -37,9 +37,9 @@ def _build(lib, mask, rate, noalloc):
         bad = torch.full((1,), -1, dtype=torch.int32, device=DEV)
         rc = lib.ua_tilelist_build_device_noalloc(m.data_ptr(), nqb, nkb, rate, *ptrs, bad.data_ptr(), st)
     else:
-        work = torch.empty(nqt + nkt + 3, dtype=torch.int32, device=DEV)
+        work = torch.empty(nqt + nkt + 7, dtype=torch.int32, device=DEV)
         rc = lib.ua_tilelist_build_device(m.data_ptr(), nqb, nkb, rate, *ptrs, work.data_ptr(), st)
-        bad = work[-1:]
+        bad = work[nqt + nkt + 2:nqt + nkt + 3]
     assert rc == 0, lib.ua_strerror(rc)
     torch.cuda.synchronize()
     return {f: out[f][:nnz.value].cpu().numpy() if f in ("col_idx", "flag", "row_idx", "cflag") else out[f].cpu().numpy()

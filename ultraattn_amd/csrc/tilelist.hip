@@ -13,7 +13,7 @@
 // per-row and per-column tile counts that the device builder otherwise keeps in the caller's
 // `work` argument.  Every GPU the library runs on holds its own copy (256 KiB) until the process
 // ends; calls on one GPU share it, so two such calls must not overlap.
-static __device__ __align__(256) int32_t scratch[UA_NOALLOC_MAX_LINES + 4];
+static __device__ __align__(256) int32_t scratch[UA_NOALLOC_MAX_LINES + 8];
 
 namespace ua {
 
@@ -25,25 +25,53 @@ __host__ __device__ __forceinline__ int tile_type(const uint8_t* mask, int nkb, 
   return a == b ? 2 : (a > b ? 1 : 0);
 }
 
-// Launch order: does row a come before row b?  Rows much longer than average
-// (len * n > 2 * nnz) first, longest first; the rest in lexicographic order of their index
-// lists, a list that is a prefix of another sorting after it; ties by row number.  Rows that
-// walk the same K/V (or Q/dO) tiles thus sit next to each other in the launch.
-__host__ __device__ __forceinline__ bool row_precedes(const int32_t* ptr, const int32_t* idx, int n, int a, int b) {
+// Launch order: does line a (a row of the CSR, or a column of the CSC) come before line b?
+//  1. Lines much longer than average (len * n > 2 * nnz) first, longest first: they cannot end
+//     up as the tail of the launch.
+//  2. The rest by their anchor index, ascending.  The anchor is the first index of the list, or
+//     the last one when `from_end`: lines that share it walk common tiles (the rows of a causal
+//     mask share their oldest keys, its columns their latest queries).
+//  3. Among those, the lines of longer block lines first (the length of a tile's block line =
+//     the list length of that block's longest tile: sub-tile rate-1 of a row block, sub-tile 0 of
+//     a column block): the short lists end the group, and a list that leaves the common part
+//     early does not run ahead of the lists that still walk it.
+//  4. Then lexicographic order of the index lists read from the anchor, a list that is a prefix
+//     (from_end: a suffix) of another sorting after it; ties by line number.  Lines that walk the
+//     same K/V (or Q/dO) tiles thus sit next to each other in the launch and share them in L2.
+__host__ __device__ __forceinline__ bool very_long(const int32_t* ptr, int n, int a) {
+  return (int64_t)(ptr[a + 1] - ptr[a]) * n > 2 * (int64_t)ptr[n];
+}
+__host__ __device__ __forceinline__ bool row_precedes(const int32_t* ptr, const int32_t* idx, int n, int rate, int longest_sub,
+                                                      bool from_end, int a, int b) {
   const int pa = ptr[a], pb = ptr[b];
   const int la = ptr[a + 1] - pa, lb = ptr[b + 1] - pb;
-  const int64_t nnz2 = 2 * (int64_t)ptr[n];
-  const bool va = (int64_t)la * n > nnz2, vb = (int64_t)lb * n > nnz2;
+  const bool va = very_long(ptr, n, a), vb = very_long(ptr, n, b);
   if (va != vb) return va;
-  if (!va) {
+  if (!va && la > 0 && lb > 0) {
+    // element t of a list, counted from its anchor
+    const int sa = from_end ? pa + la - 1 : pa, sb = from_end ? pb + lb - 1 : pb, step = from_end ? -1 : 1;
+    const int fa = idx[sa], fb = idx[sb];
+    if (fa != fb) return fa < fb;
+    const int ra = a / rate * rate + longest_sub, rb = b / rate * rate + longest_sub;
+    const int ba = ptr[ra + 1] - ptr[ra], bb = ptr[rb + 1] - ptr[rb];
+    if (ba != bb) return ba > bb;
     const int m = la < lb ? la : lb;
-    for (int t = 0; t < m; ++t) {
-      const int ca = idx[pa + t], cb = idx[pb + t];
+    for (int t = 1; t < m; ++t) {
+      const int ca = idx[sa + t * step], cb = idx[sb + t * step];
       if (ca != cb) return ca < cb;
     }
   }
   if (la != lb) return la > lb;
   return a < b;
+}
+// Which end anchors the order of one side: the one with FEWER distinct values over the lines that
+// rule 2 applies to (more lines share it); the start on a tie.
+inline bool anchor_from_end(const int32_t* ptr, const int32_t* idx, int n) {
+  std::vector<int32_t> first, last;
+  for (int i = 0; i < n; ++i)
+    if (ptr[i + 1] > ptr[i] && !very_long(ptr, n, i)) { first.push_back(idx[ptr[i]]); last.push_back(idx[ptr[i + 1] - 1]); }
+  auto distinct = [](std::vector<int32_t>& v) { std::sort(v.begin(), v.end()); return std::unique(v.begin(), v.end()) - v.begin(); };
+  return distinct(last) < distinct(first);
 }
 
 static int check_mask(const uint8_t* mask, int nqb, int nkb, int rate) {
@@ -105,8 +133,9 @@ __global__ __launch_bounds__(64 * kWavesPerGroup) void tl_count_kernel(const uin
 // check: a single workgroup counts the mask entries that are not a Block_Type (> 2); the
 // builder treats them as EMPTY, and the count lets the caller detect them after the stream
 // has been synchronised (the host builder returns UA_ERR_MASK for the same input).
-__global__ __launch_bounds__(1024) void tl_check_kernel(const uint8_t* mask, int64_t n, int32_t* n_invalid) {
+__global__ __launch_bounds__(1024) void tl_check_kernel(const uint8_t* mask, int64_t n, int32_t* n_invalid, int32_t* anchor_cnt) {
   __shared__ int32_t part[16];
+  if (threadIdx.x < 4) anchor_cnt[threadIdx.x] = 0;      // counted by tl_anchor_kernel, later in the stream
   int bad = 0;
   for (int64_t i = threadIdx.x; i < n; i += 1024) bad += mask[i] > 2;
   bad = wave_sum(bad);
@@ -175,10 +204,38 @@ __global__ __launch_bounds__(64 * kWavesPerGroup) void tl_fill_kernel(const uint
   }
 }
 
+// anchor: number of distinct first and of distinct last indices over the lines of each side that are
+// neither empty nor very long -> anchor_cnt[0..1] for the rows, [2..3] for the columns.  One workgroup
+// per line; the line counts if no earlier line of its side holds the same value.
+__global__ __launch_bounds__(256) void tl_anchor_kernel(const int32_t* qptr, const int32_t* qidx, int nq,
+                                                        const int32_t* kptr, const int32_t* kidx, int nk, int32_t* anchor_cnt) {
+  __shared__ int dup_s[2];
+  const int t = blockIdx.x;
+  const int32_t* ptr = t < nq ? qptr : kptr;
+  const int32_t* idx = t < nq ? qidx : kidx;
+  const int n = t < nq ? nq : nk;
+  const int i = t < nq ? t : t - nq;
+  if (ptr[i + 1] == ptr[i] || very_long(ptr, n, i)) return;
+  if (threadIdx.x < 2) dup_s[threadIdx.x] = 0;
+  __syncthreads();
+  const int first = idx[ptr[i]], last = idx[ptr[i + 1] - 1];
+  bool df = false, dl = false;
+  for (int j = threadIdx.x; j < i; j += 256) {
+    if (ptr[j + 1] == ptr[j] || very_long(ptr, n, j)) continue;
+    df |= idx[ptr[j]] == first;
+    dl |= idx[ptr[j + 1] - 1] == last;
+  }
+  if (df) dup_s[0] = 1;
+  if (dl) dup_s[1] = 1;
+  __syncthreads();
+  if (threadIdx.x < 2 && !dup_s[threadIdx.x]) atomicAdd(&anchor_cnt[(t < nq ? 0 : 2) + threadIdx.x], 1);
+}
+
 // order: rank of a line = number of lines that precede it; one workgroup per line, its threads
 // share the comparisons.
 __global__ __launch_bounds__(256) void tl_order_kernel(const int32_t* qptr, const int32_t* qidx, int nq, int32_t* q_order,
-                                                       const int32_t* kptr, const int32_t* kidx, int nk, int32_t* k_order) {
+                                                       const int32_t* kptr, const int32_t* kidx, int nk, int32_t* k_order, int rate,
+                                                       const int32_t* anchor_cnt) {
   __shared__ int rank_s;
   const int t = blockIdx.x;
   const int32_t* ptr = t < nq ? qptr : kptr;
@@ -186,10 +243,13 @@ __global__ __launch_bounds__(256) void tl_order_kernel(const int32_t* qptr, cons
   const int n = t < nq ? nq : nk;
   int32_t* order = t < nq ? q_order : k_order;
   const int i = t < nq ? t : t - nq;
+  const int longest_sub = t < nq ? rate - 1 : 0;
+  const int32_t* cnt = anchor_cnt + (t < nq ? 0 : 2);
+  const bool from_end = cnt[1] < cnt[0];
   if (threadIdx.x == 0) rank_s = 0;
   __syncthreads();
   int rank = 0;
-  for (int j = threadIdx.x; j < n; j += 256) rank += (j != i) && row_precedes(ptr, idx, n, j, i);
+  for (int j = threadIdx.x; j < n; j += 256) rank += (j != i) && row_precedes(ptr, idx, n, rate, longest_sub, from_end, j, i);
   rank = wave_sum(rank);
   if ((threadIdx.x & 63) == 0) atomicAdd(&rank_s, rank);
   __syncthreads();
@@ -248,9 +308,10 @@ extern "C" int ua_tilelist_build(const uint8_t* block_mask, int n_qblocks, int n
       row_idx[pos] = qt; cflag[pos] = flag[i];
     }
   std::iota(q_order, q_order + nqt, 0);
-  std::sort(q_order, q_order + nqt, [&](int32_t a, int32_t b) { return row_precedes(row_ptr, col_idx, nqt, a, b); });
+  const bool q_end = anchor_from_end(row_ptr, col_idx, nqt), k_end = anchor_from_end(col_ptr, row_idx, nkt);
+  std::sort(q_order, q_order + nqt, [&](int32_t a, int32_t b) { return row_precedes(row_ptr, col_idx, nqt, rate, rate - 1, q_end, a, b); });
   std::iota(k_order, k_order + nkt, 0);
-  std::sort(k_order, k_order + nkt, [&](int32_t a, int32_t b) { return row_precedes(col_ptr, row_idx, nkt, a, b); });
+  std::sort(k_order, k_order + nkt, [&](int32_t a, int32_t b) { return row_precedes(col_ptr, row_idx, nkt, rate, 0, k_end, a, b); });
   return UA_OK;
 }
 
@@ -263,16 +324,20 @@ static int build_device_impl(const uint8_t* block_mask, int n_qblocks, int n_kbl
   const int nqt = n_qblocks * rate, nkt = n_kblocks * rate;
   int32_t* qcnt = work;
   int32_t* kcnt = work + nqt + 1;
-  hipLaunchKernelGGL(tl_check_kernel, dim3(1), dim3(1024), 0, st, block_mask, (int64_t)n_qblocks * n_kblocks, n_invalid);
+  int32_t* anchor_cnt = work + nqt + nkt + 3;
+  hipLaunchKernelGGL(tl_check_kernel, dim3(1), dim3(1024), 0, st, block_mask, (int64_t)n_qblocks * n_kblocks, n_invalid, anchor_cnt);
   const int blocks = (nqt + nkt + kWavesPerGroup - 1) / kWavesPerGroup;
   hipLaunchKernelGGL(tl_count_kernel, dim3(blocks), dim3(64 * kWavesPerGroup), 0, st, block_mask, n_qblocks, n_kblocks, rate, qcnt, kcnt);
   hipLaunchKernelGGL(tl_scan_kernel, dim3(1), dim3(1024), 0, st, (const int32_t*)qcnt, nqt, row_ptr);
   hipLaunchKernelGGL(tl_scan_kernel, dim3(1), dim3(1024), 0, st, (const int32_t*)kcnt, nkt, col_ptr);
   hipLaunchKernelGGL(tl_fill_kernel, dim3(blocks), dim3(64 * kWavesPerGroup), 0, st, block_mask, n_qblocks, n_kblocks, rate,
                      (const int32_t*)row_ptr, col_idx, flag, (const int32_t*)col_ptr, row_idx, cflag);
+  hipLaunchKernelGGL(tl_anchor_kernel, dim3(nqt + nkt), dim3(256), 0, st,
+                     (const int32_t*)row_ptr, (const int32_t*)col_idx, nqt,
+                     (const int32_t*)col_ptr, (const int32_t*)row_idx, nkt, anchor_cnt);
   hipLaunchKernelGGL(tl_order_kernel, dim3(nqt + nkt), dim3(256), 0, st,
                      (const int32_t*)row_ptr, (const int32_t*)col_idx, nqt, q_order,
-                     (const int32_t*)col_ptr, (const int32_t*)row_idx, nkt, k_order);
+                     (const int32_t*)col_ptr, (const int32_t*)row_idx, nkt, k_order, rate, (const int32_t*)anchor_cnt);
   return hipGetLastError() == hipSuccess ? UA_OK : UA_ERR_LAUNCH;
 }
 

@@ -112,15 +112,15 @@ def build_tile_list_device(block_mask_dev, block: int = 512, nnz: Optional[int] 
     out = dict(row_ptr=torch.empty(nqt + 1, **i32), col_idx=torch.empty(alloc, **i32), flag=torch.empty(alloc, **u8),
                col_ptr=torch.empty(nkt + 1, **i32), row_idx=torch.empty(alloc, **i32), cflag=torch.empty(alloc, **u8),
                q_order=torch.empty(nqt, **i32), k_order=torch.empty(nkt, **i32))
-    work = torch.empty(nqt + nkt + 3, **i32)
+    work = torch.empty(nqt + nkt + 7, **i32)
     lib = _lib.load()
     with torch.cuda.device(dev):
         st = torch.cuda.current_stream().cuda_stream
         _lib.check(lib.ua_tilelist_build_device(m.data_ptr(), nqb, nkb, rate,
                                                 *[out[n].data_ptr() for n in _HOST_FIELDS],
                                                 work.data_ptr(), st), "ua_tilelist_build_device")
-    if check and int(work[-1].item()) != 0:
-        raise ValueError(f"block mask holds {int(work[-1].item())} entries other than 0 (EMPTY), 1 (FULL), 2 (CAUSAL)")
+    if check and int(work[nqt + nkt + 2].item()) != 0:
+        raise ValueError(f"block mask holds {int(work[nqt + nkt + 2].item())} entries other than 0 (EMPTY), 1 (FULL), 2 (CAUSAL)")
     for n in ("col_idx", "flag", "row_idx", "cflag"):
         out[n] = out[n][:cap]
     return out
