@@ -311,7 +311,7 @@ def run_mask_builder(name, steps):
     ms = e0.elapsed_time(e1) / steps
     nbytes = mask.size + 2 * host.nnz * 5 + 4 * (2 * (host.n_qtiles + host.n_ktiles) + 2)
     return {"workload": name, "ms": ms, "bytes": nbytes, "gbps": nbytes / ms / 1e6, "nnz_tiles": host.nnz,
-            "matches_host_builder": same, "note": "latency-bound: 4 dependent launches over a few MB"}
+            "matches_host_builder": same, "note": "latency-bound: 8 dependent launches over a few MB"}
 
 
 def run_cols_gather(steps):

@@ -19,8 +19,10 @@
  *    the transposed CSC over key tiles.  flag 0 = full tile, 1 = causal tile (key j visible to
  *    query i iff j <= i on tile-local indices; such tiles sit on the mask's diagonal,
  *    orchestrated_attn/orchestrated_attn_impl.py:91).  `*_order` is a permutation of the tile
- *    rows (columns) giving the launch order: rows much longer than average first, the rest in
- *    lexicographic order of their index lists so that rows sharing K/V tiles run together.
+ *    rows (columns) giving the launch order, a performance hint that does not change results:
+ *    rows much longer than average first, the rest grouped by their first (or, where that is
+ *    shared by more rows, last) index, longer block rows first, then lexicographically, so that
+ *    rows sharing K/V tiles run together.
  *    `nnz` is the number of entries of col_idx/flag (row_idx/cflag): the kernels clamp every
  *    list bound to it, and only an empty list (nnz = 0) may pass NULL for those arrays.
  *  - Every function returns 0 (UA_OK) or a negative UA_ERR_* code; ua_strerror() names it.
