@@ -54,6 +54,9 @@ extern "C" {
 #define UA_MAX_PARTS 16    /* most partial outputs one ua_merge call combines */
 #define UA_NOALLOC_MAX_LINES 65532   /* most query tiles + key tiles of ua_tilelist_build_device_noalloc */
 
+/* 100 * major + minor.  102: `nnz` argument of the attention entry points, ua_merge_update, the
+ * no-allocation builder, `work` of ua_tilelist_build_device grown to n_qtiles + n_ktiles + 7.  */
+#define UA_VERSION 102
 int ua_version(void);
 const char *ua_strerror(int rc);
 

@@ -29,7 +29,8 @@ def test_header_symbols_are_exported(lib):
     for n in names:
         assert hasattr(raw, n), f"{n} declared in include/ultraattn.h but not exported"
     assert sorted(_lib.SIGNATURES) == names, "python binding and header disagree"
-    assert lib.ua_version() >= 100
+    header = open(os.path.join(ROOT, "include", "ultraattn.h")).read()
+    assert lib.ua_version() == int(re.search(r"#define UA_VERSION (\d+)", header).group(1)) >= 102
 
 
 def test_argument_checks_without_gpu(lib):

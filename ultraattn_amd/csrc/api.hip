@@ -23,7 +23,7 @@ int check_device() {
 
 }  // namespace ua
 
-extern "C" int ua_version(void) { return 100; }
+extern "C" int ua_version(void) { return UA_VERSION; }
 
 extern "C" const char* ua_strerror(int rc) {
   switch (rc) {
