@@ -20,6 +20,10 @@ FIELDS = ("row_ptr", "col_idx", "flag", "col_ptr", "row_idx", "cflag", "q_order"
     (lambda: masks.config_global_local(), 512), (lambda: masks.config_streaming_shard(), 512),
     (lambda: masks.canonical_block_table(3), 1024), (lambda: np.zeros((2, 3), np.uint8), 256),
     (lambda: np.random.RandomState(3).randint(0, 3, size=(7, 5)).astype(np.uint8), 384),
+    (lambda: np.random.RandomState(4).randint(0, 2, size=(33, 17)).astype(np.uint8), 128),
+    (lambda: np.tril(np.random.RandomState(5).randint(0, 2, size=(24, 24))).astype(np.uint8), 256),
+    (lambda: np.triu(np.random.RandomState(6).randint(0, 3, size=(19, 31))).astype(np.uint8), 512),
+    (lambda: masks.canonical_block_table(0), 512), (lambda: masks.canonical_block_table(1), 256),
 ])
 def test_device_builder_bit_exact(make, block):
     m = make()
