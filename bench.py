@@ -570,7 +570,32 @@ def cpu_baseline():
     return {"value": F / best / 1e12, "unit": "TFLOP/s", "cores": torch.get_num_threads(), "kind": "port",
             "sample": "config 1 whole: B=1 S=8192 Nh=8 d=128 fp32 causal 16x16 blocks of 512, forward, "
                       f"{len(timed)} runs, min {best:.3f} s, median {sorted(timed)[len(timed) // 2]:.3f} s",
-            "affinity_cores": len(os.sched_getaffinity(0)), "flops": F}
+            "affinity_cores": len(os.sched_getaffinity(0)), "flops": F,
+            "parity": config1_parity(ao, mask, q, k, v)}
+
+
+def config1_parity(ao, mask, q, k, v):
+    """The HIP path against the CPU block loop on config 1's workload (the same bf16-rounded q, k, v
+    and a seeded dO on both sides): largest deviations of O, LSE, dQ, dK, dV."""
+    import torch
+    from ultraattn_amd import ops
+    from ultraattn_amd.tilelist import build_tile_list
+    g = torch.Generator().manual_seed(1)
+    do = torch.randn(q.shape, generator=g, dtype=torch.float32)
+    qb, kb, vb, dob = (t.to(torch.bfloat16) for t in (q, k, v, do))
+    ro, rl = ao.block_loop_fwd(qb, kb, vb, mask, BLOCK, SCALE)
+    rq, rk, rv = ao.block_loop_bwd(dob, qb, kb, vb, ro, rl, mask, BLOCK, SCALE)
+    tl = build_tile_list(mask, BLOCK)
+    qd, kd, vd, dod = (t.to("cuda:0") for t in (qb, kb, vb, dob))
+    o, lse = ops.bsa_fwd(qd, kd, vd, tl, SCALE)
+    dq, dk, dv = ops.bsa_bwd(dod, qd, kd, vd, o, lse, tl, SCALE)
+    torch.cuda.synchronize()
+    err = lambda a, b: (a.detach().float().cpu() - b.float()).abs().max().item()
+    lse_c, rl = lse.cpu().double(), rl.double()
+    return {"workload": "config 1 (S=8192, Nh=8, 16x16 causal blocks), bf16-rounded inputs, against the CPU block loop",
+            "o_max_abs": err(o, ro), "lse_max_rel": ((lse_c - rl).abs() / rl.abs().clamp_min(1.0)).max().item(),
+            "dq_max_abs": err(dq, rq), "dk_max_abs": err(dk, rk), "dv_max_abs": err(dv, rv),
+            "bounds": {"o_dq_dk_dv_max_abs": 2e-2, "lse_max_rel": 1e-3}}
 
 
 def main():
@@ -671,6 +696,7 @@ def main():
     log(json.dumps(out["mfma_probe"]))
     if not a.no_cpu:
         out["cpu_baseline"] = cpu_baseline()
+        out["parity"] = out["cpu_baseline"]["parity"]          # the same object, at the top level too
         log(json.dumps(out["cpu_baseline"]))
     print(json.dumps(out), flush=True)
 
