@@ -678,7 +678,7 @@ def main():
            "config": {"workload": {"c2": "causal 32k (config 2), forward", "c3": "strided 128k (config 3), forward+backward",
                                    "c4": "global+local 128k (config 4), forward+backward",
                                    "c5": "streaming shard 64k x 512k (config 5), 4 forward kernel tiles + merge"}[a.workload],
-                      "batch": 1, "heads": HEADS, "head_dim": 128, "block": BLOCK, "tile": 128,
+                      "seed": 0, "batch": 1, "heads": HEADS, "head_dim": 128, "block": BLOCK, "tile": 128,
                       "seq_q": int(workload_mask(a.workload).shape[0]) * BLOCK,
                       "seq_kv": int(workload_mask(a.workload).shape[1]) * BLOCK},
            "frac_of_bf16_mfma_peak": value / peak, "peak_tflops": peak, "detail": main_res,
