@@ -133,7 +133,8 @@ def build_tile_list(block_table: np.ndarray, rate: int) -> Dict[str, np.ndarray]
 def launch_order(ptr: np.ndarray, idx: np.ndarray, rate: int, longest_sub: int) -> np.ndarray:
     """Launch order of the rows of a CSR (``longest_sub = rate - 1``) or the columns of a CSC
     (``longest_sub = 0``).  Rows much longer than average (length * n_rows > 2 * nnz) come first,
-    longest first, so that they cannot end up as the tail of the launch.  The others are ordered by
+    so that they cannot end up as the tail of the launch, longest block line first and then
+    lexicographically from the anchor as below.  The others are ordered by
     their anchor index: the first index of the list, or the last one if the last indices take
     fewer distinct values than the first ones over these rows (the lists are then read backwards
     below); then by the length of their block line, longest first (measured as the list length of
@@ -149,14 +150,15 @@ def launch_order(ptr: np.ndarray, idx: np.ndarray, rate: int, longest_sub: int) 
 
     def key(i):
         lst = lists[i]
-        if len(lst) * n > 2 * nnz:
-            return (0, (-len(lst),), i)
         if not lst:
             return (2, (), i)
         ref = i // rate * rate + longest_sub
+        block_len = int(ptr[ref + 1] - ptr[ref])
         if from_end:
             lst = lst[::-1]
-        return (1, (lst[0], -int(ptr[ref + 1] - ptr[ref])) + lst[1:] + (inf,), i)
+        if len(lst) * n > 2 * nnz:
+            return (0, (-block_len,) + lst + (inf,), i)
+        return (1, (lst[0], -block_len) + lst[1:] + (inf,), i)
     return np.array(sorted(range(n), key=key), dtype=np.int32).reshape(-1)
 
 

@@ -26,8 +26,8 @@ __host__ __device__ __forceinline__ int tile_type(const uint8_t* mask, int nkb, 
 }
 
 // Launch order: does line a (a row of the CSR, or a column of the CSC) come before line b?
-//  1. Lines much longer than average (len * n > 2 * nnz) first, longest first: they cannot end
-//     up as the tail of the launch.
+//  1. Lines much longer than average (len * n > 2 * nnz) first, so that they cannot end up as
+//     the tail of the launch; among them the longer block lines first (see 3), then as in 4.
 //  2. The rest by their anchor index, ascending.  The anchor is the first index of the list, or
 //     the last one when `from_end`: lines that share it walk common tiles (the rows of a causal
 //     mask share their oldest keys, its columns their latest queries).
@@ -47,14 +47,19 @@ __host__ __device__ __forceinline__ bool row_precedes(const int32_t* ptr, const 
   const int la = ptr[a + 1] - pa, lb = ptr[b + 1] - pb;
   const bool va = very_long(ptr, n, a), vb = very_long(ptr, n, b);
   if (va != vb) return va;
-  if (!va && la > 0 && lb > 0) {
+  if (la > 0 && lb > 0) {
     // element t of a list, counted from its anchor
     const int sa = from_end ? pa + la - 1 : pa, sb = from_end ? pb + lb - 1 : pb, step = from_end ? -1 : 1;
     const int fa = idx[sa], fb = idx[sb];
-    if (fa != fb) return fa < fb;
     const int ra = a / rate * rate + longest_sub, rb = b / rate * rate + longest_sub;
     const int ba = ptr[ra + 1] - ptr[ra], bb = ptr[rb + 1] - ptr[rb];
-    if (ba != bb) return ba > bb;
+    if (va) {                       // rule 1: block-line length decides before the anchor
+      if (ba != bb) return ba > bb;
+      if (fa != fb) return fa < fb;
+    } else {
+      if (fa != fb) return fa < fb;
+      if (ba != bb) return ba > bb;
+    }
     const int m = la < lb ? la : lb;
     for (int t = 1; t < m; ++t) {
       const int ca = idx[sa + t * step], cb = idx[sb + t * step];
