@@ -67,6 +67,18 @@ CASES = [("strided 128k rows", masks.config_strided, "q", 0.12), ("strided 128k 
          ("streaming shard rows", masks.config_streaming_shard, "q", 0.06)]
 
 
+def _shard_key_range(part):
+    """One of the four key-range kernel tiles of the streaming shard (as bench.py splits it)."""
+    mask = masks.config_streaming_shard()
+    cols = np.array_split(np.nonzero(mask.any(0))[0], 4)[part]
+    sub = np.zeros_like(mask)
+    sub[:, cols] = mask[:, cols]
+    return sub
+
+
+CASES += [(f"streaming shard, key range {p} of 4, rows", (lambda p=p: _shard_key_range(p)), "q", 0.08) for p in range(4)]
+
+
 @pytest.mark.parametrize("name,make,side,bound", CASES, ids=[c[0] for c in CASES])
 def test_launch_order_keeps_shared_tiles_in_cache(name, make, side, bound):
     tl = build_tile_list(make(), block=512)
@@ -76,4 +88,4 @@ def test_launch_order_keeps_shared_tiles_in_cache(name, make, side, bound):
     ref_miss, _ = simulate(lists, lexicographic(lists))
     assert miss <= bound, (name, miss)
     assert miss <= ref_miss + 0.005, (name, miss, ref_miss)
-    assert occupancy >= 0.985, (name, occupancy)
+    assert occupancy >= (0.985 if "key range" not in name else 0.95), (name, occupancy)
