@@ -25,10 +25,16 @@
  *    rows sharing K/V tiles run together.
  *    `nnz` is the number of entries of col_idx/flag (row_idx/cflag): the kernels clamp every
  *    list bound to it, and only an empty list (nnz = 0) may pass NULL for those arrays.
+ *    flag / cflag are read one aligned 32-bit word at a time: they must start on a 4-byte boundary
+ *    (else UA_ERR_ALIGN) and be readable up to the next multiple of 4 bytes after entry nnz-1, i.e.
+ *    allocate (nnz + 3) / 4 * 4 bytes; the padding bytes are never interpreted.
  *  - Every function returns 0 (UA_OK) or a negative UA_ERR_* code; ua_strerror() names it.
  *    No exceptions cross this boundary and nothing aborts.
- *  - Functions hold no mutable global state and may be called from several host threads on
- *    different streams.
+ *  - Functions may be called from several host threads on different streams.  The only state
+ *    the library keeps is per-device and write-once (the device check's result and the address of
+ *    the fixed scratch), set by ua_init() or by the first call on a device; the one exception is the
+ *    CONTENT of that scratch, which ua_tilelist_build_device_noalloc calls on one GPU share (see
+ *    there).
  */
 #ifndef ULTRAATTN_H
 #define ULTRAATTN_H
@@ -56,9 +62,18 @@ extern "C" {
 
 /* 100 * major + minor.  102: `nnz` argument of the attention entry points, ua_merge_update, the
  * no-allocation builder, `work` of ua_tilelist_build_device grown to n_qtiles + n_ktiles + 7.  */
-#define UA_VERSION 102
+#define UA_VERSION 103
 int ua_version(void);
 const char *ua_strerror(int rc);
+
+/* No counterpart in the reference.  Resolves, for the CURRENT device, everything the entry points
+ * otherwise look up on their first call there: the device's architecture (hipGetDeviceProperties)
+ * and the address of the library's fixed scratch (hipGetSymbolAddress, which also loads the code
+ * object).  Those lookups are not legal while a stream is being captured into a HIP graph, so a
+ * caller that captures a FIRST call of any entry point calls ua_init() once per device
+ * beforehand, outside capture.  Allocates nothing; idempotent; UA_ERR_DEVICE if the device is not
+ * gfx950.                                                                                      */
+int ua_init(void);
 
 /* ---- block mask -> active-tile list (host) ------------------------------------------------
  * Replaces the reference's Python enumeration of Comp_Kernels from a block table:
@@ -92,11 +107,12 @@ int ua_tilelist_build_device(const uint8_t *block_mask, int n_qblocks, int n_kbl
 /* No counterpart in the reference.  For callers that cannot allocate device memory (code under
  * HIP graph capture, tight serving loops, harnesses that forbid it): the same builder as
  * ua_tilelist_build_device with the `work` scratch taken from a fixed array inside the library
- * (256 KiB + 32 B per GPU, held until the process ends) instead of from the caller.  Limit:
+ * (256 KiB + 16 B per GPU, held until the process ends) instead of from the caller.  Limit:
  * n_qtiles + n_ktiles <= UA_NOALLOC_MAX_LINES, else UA_ERR_TOO_LARGE.  `n_invalid` (device,
  * may be NULL) receives the number of mask entries that are not 0, 1 or 2.  It calls no
  * hipMalloc/hipFree.  All calls on one GPU share the array: calls that overlap in time on the
- * same GPU (different streams or threads) race; serialise them.                             */
+ * same GPU (different streams or threads) race; serialise them.  The first call on a device looks
+ * up the scratch address (see ua_init): under graph capture call ua_init() first.              */
 int ua_tilelist_build_device_noalloc(const uint8_t *block_mask, int n_qblocks, int n_kblocks, int rate,
                                      int32_t *row_ptr, int32_t *col_idx, uint8_t *flag,
                                      int32_t *col_ptr, int32_t *row_idx, uint8_t *cflag,
@@ -164,8 +180,9 @@ int ua_merge(const void *const *o_parts, const float *const *lse_parts, int n_pa
  * pointer offset), statistics fp32 in either the reference's running layout [B, S, Nh, 1]
  * (strides S*Nh, Nh, 1) or the kernels' [B, Nh, S] (strides Nh*S, 1, S).  `*_is_fp32` select
  * fp32 or bf16 rows (the reference's running `out` turns fp32 after its first update).
- * new_out / new_lse may be exactly out / lse (the slice_ path: same pointer, same strides) or
- * buffers that do not overlap them; partial overlap is undefined.  Row strides must keep rows
+ * new_out / new_lse may be exactly out / lse (the slice_ path: same pointer, then the same element
+ * type and strides are required, else UA_ERR_SHAPE) or buffers that do not overlap them; partial
+ * overlap is undefined.  Row strides must keep rows
  * 16-byte aligned (multiples of 8 bf16 / 4 fp32 elements).                                   */
 int ua_merge_update(const void *out, const float *lse, const void *block_out, const float *block_lse,
                     void *new_out, float *new_lse, int batch, int n_rows, int n_heads, int head_dim,
@@ -173,6 +190,25 @@ int ua_merge_update(const void *out, const float *lse, const void *block_out, co
                     const int64_t *out_strides, const int64_t *lse_strides,
                     const int64_t *block_out_strides, const int64_t *block_lse_strides,
                     const int64_t *new_out_strides, const int64_t *new_lse_strides, void *stream);
+
+/* ---- accumulation of partial gradients -------------------------------------------------------
+ * The reduce() of the gradient packs that the reference leaves as stubs
+ * (orchestrated_attn/utils.py:260-262, 296-298: `self.data.add_(other.data)` commented out), with
+ * the accumulation its ring executor specifies (ring_flash_attn/ring_flash_attn.py:110-118:
+ * partial dq/dk/dv are added into fp32 buffers and cast to bf16 once).
+ * ua_grad_accumulate: one step of a running sum over `n` contiguous elements (n a multiple of 8),
+ *   acc != NULL, init_from_out == 0 :  acc += partial;  out = bf16(acc) when out != NULL
+ *   acc != NULL, init_from_out != 0 :  acc  = float(out) + partial;  out = bf16(acc)   (first step)
+ *   acc == NULL                     :  out  = bf16(float(out) + partial)
+ *   acc fp32, partial and out bf16; one pass (read acc + partial, write acc + out).
+ * ua_grad_sum: out = bf16(scale * sum_p parts[p]) over n_parts (1..UA_MAX_PARTS) partial gradients
+ *   in one pass.  `parts` is a HOST array of DEVICE pointers to contiguous
+ *   [batch, seqlen, n_heads, 128] arrays, fp32 when parts_fp32 != 0, else bf16; `out` is bf16 and
+ *   takes (batch, token, head) element strides (multiples of 8).                                */
+int ua_grad_accumulate(float *acc, const void *partial, void *out, int64_t n, int init_from_out, void *stream);
+int ua_grad_sum(const void *const *parts, int n_parts, int parts_fp32, void *out,
+                int batch, int seqlen, int n_heads, int head_dim, const int64_t *out_strides,
+                float scale, void *stream);
 
 /* ---- column-buffer layout changes around a fused rectangle -----------------------------------
  * Replace the two torch transpose+contiguous copies of the X x Y path:

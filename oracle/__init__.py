@@ -28,6 +28,8 @@ Pinning status (what each function is checked against, see tests/test_oracle_*.p
                         finite differences, row-sum identities.                       PINNED
 * ``update_out_and_lse`` / ``merge_partials`` : torch.logaddexp, single-pass result over the
                         union of key sets, equal-LSE average, -inf identity.          PINNED
+* ``accumulate_gradients`` : left-to-right fp32 sum equals the fp64 sum rounded to fp32 on
+                        exactly representable inputs; differs from a bf16 running sum.    PINNED
 * ``tilelist``        : brute-force element mask, counts derived independently,
                         reference-held mask strings and allocation logs.              PINNED
 * ``layout_oracle``   : explicit index loops, the reference's torch view/transpose chain,

@@ -147,6 +147,17 @@ def merge_partials(outs: Sequence[torch.Tensor], lses: Sequence[torch.Tensor], d
 # the block loop: what orchestrated_attn / hierarchy_attn execute on one device
 # --------------------------------------------------------------------------------------
 
+def accumulate_gradients(parts: Sequence[torch.Tensor]):
+    """The gradient accumulation of ``ring_flash_attn/ring_flash_attn.py:110-118``: the first
+    partial is converted to fp32 (``dq = block_dq_buffer.to(torch.float32)``), every later one is
+    added into that fp32 buffer (``dq += block_dq_buffer``), and the result is cast to the
+    partials' dtype once (``:135``).  Returns (fp32 sum, its cast)."""
+    acc = parts[0].to(torch.float32)
+    for p in parts[1:]:
+        acc = acc + p            # bf16 -> fp32 promotion, as `dq += block` does
+    return acc, acc.to(parts[0].dtype)
+
+
 def block_loop_fwd(q, k, v, block_table: np.ndarray, block: int, scale: float,
                    dtype=torch.float32, q_block_offset: int = 0):
     """Forward over a block table with values 0 EMPTY / 1 FULL / 2 CAUSAL

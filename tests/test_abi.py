@@ -76,6 +76,26 @@ def test_argument_checks_without_gpu(lib):
     assert lib.ua_merge_update(*ok, 1, 0, 1, 128, 0, 0, 0, s, ls, s, ls, s, ls, None) == -2
     odd = (ctypes.c_int64 * 3)(128 * 128, 132, 128)          # bf16 rows need strides in multiples of 8
     assert lib.ua_merge_update(*ok, 1, 16, 1, 128, 0, 0, 0, odd, ls, s, ls, s, ls, None) == -4
+    # the same pointer for out and new_out needs the same element type and strides
+    s2 = (ctypes.c_int64 * 3)(128 * 256, 256, 128)
+    assert lib.ua_merge_update(buf, buf, buf + 64, buf, buf, buf, 1, 16, 1, 128, 0, 0, 1, s, ls, s, ls, s, ls, None) == -2
+    assert lib.ua_merge_update(buf, buf, buf + 64, buf, buf, buf, 1, 16, 1, 128, 0, 0, 0, s, ls, s, ls, s2, ls, None) == -2
+    # flag arrays are read as aligned 32-bit words
+    assert lib.ua_bsa_fwd(buf, buf, buf, buf, buf, buf, buf, buf + 1, buf, 1, 1, 1, 1, 1, 128, s, s, s, s, 0.1, None) == -4
+    assert lib.ua_bsa_bwd_dq(buf, buf, buf, buf, buf, buf, buf, buf, buf, buf + 2, buf, 1, 1, 1, 1, 1, 128,
+                             s, s, s, s, s, 0.1, None) == -4
+    # gradient reductions
+    assert lib.ua_grad_accumulate(buf, None, buf, 64, 0, None) == -1
+    assert lib.ua_grad_accumulate(None, buf, None, 64, 0, None) == -1
+    assert lib.ua_grad_accumulate(None, buf, buf, 64, 1, None) == -1      # init_from_out needs an accumulator
+    assert lib.ua_grad_accumulate(buf, buf, buf, 0, 0, None) == -2
+    assert lib.ua_grad_accumulate(buf, buf, buf, 60, 0, None) == -4
+    assert lib.ua_grad_accumulate(buf, buf + 2, buf, 64, 0, None) == -4
+    arr1 = (ctypes.c_void_p * 17)(*([buf] * 17))
+    assert lib.ua_grad_sum(arr1, 17, 0, buf, 1, 16, 1, 128, s, 1.0, None) == -3
+    assert lib.ua_grad_sum(arr1, 2, 0, buf, 1, 16, 1, 64, s, 1.0, None) == -3
+    assert lib.ua_grad_sum(arr1, 2, 0, buf, 1, 0, 1, 128, s, 1.0, None) == -2
+    assert lib.ua_grad_sum(None, 2, 0, buf, 1, 16, 1, 128, s, 1.0, None) == -1
     # device tile-list builders: NULL, sizes, and the no-allocation variant's limit on the number of lines
     args = (buf,) * 8
     assert lib.ua_tilelist_build_device(buf, 1, 1, 4, *args, None, None) == -1

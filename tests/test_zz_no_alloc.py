@@ -71,3 +71,48 @@ def test_noalloc_builder_rejects_what_its_scratch_cannot_hold(lib):
     rc = lib.ua_tilelist_build_device_noalloc(p, 10000, 10000, 4, p, p, p, p, p, p, p, p, None, st)
     assert rc == -8 and b"scratch" in lib.ua_strerror(rc)
     assert lib.ua_tilelist_build_device_noalloc(p, 1, 1, 1, p, p, p, p, p, p, p, None, None, st) == -1
+
+
+def test_noalloc_builder_leaves_device_memory_alone_and_runs_under_capture(lib):
+    """The second and later calls must not change the device's free memory, and after ua_init()
+    (which resolves the per-device lookups outside capture) a call can be captured into a HIP
+    graph: every replay rebuilds the lists of whatever mask is in the input buffer."""
+    assert lib.ua_init() == 0 and lib.ua_init() == 0              # idempotent
+    a = masks.config_strided(16, 2, 4)
+    b = masks.config_global_local(16, 2, 1)
+    rate = 2
+    nqt = nkt = 16 * rate
+    cap = nqt * nkt
+    m = torch.from_numpy(a).to(DEV)
+    out = _buffers(nqt, nkt, cap)
+    bad = torch.zeros(1, dtype=torch.int32, device=DEV)
+    ptrs = [out[f].data_ptr() for f in FIELDS]
+    side = torch.cuda.Stream()
+    call = lambda st: lib.ua_tilelist_build_device_noalloc(m.data_ptr(), 16, 16, rate, *ptrs, bad.data_ptr(), st)
+    with torch.cuda.stream(side):
+        assert call(side.cuda_stream) == 0                        # warm, eager
+    torch.cuda.synchronize()
+    free0 = torch.cuda.mem_get_info()[0]
+    alloc0 = torch.cuda.memory_allocated()
+    with torch.cuda.stream(side):
+        for _ in range(3):
+            assert call(side.cuda_stream) == 0
+    torch.cuda.synchronize()
+    assert torch.cuda.mem_get_info()[0] == free0 and torch.cuda.memory_allocated() == alloc0
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        assert call(torch.cuda.current_stream().cuda_stream) == 0
+    for mask in (b, a, b):
+        m.copy_(torch.from_numpy(mask))
+        for f in FIELDS:
+            out[f].fill_(77)
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        want, _ = _build(lib, mask, rate, noalloc=False)
+        nnz = want["col_idx"].shape[0]
+        for f in FIELDS:
+            got = out[f].cpu().numpy()
+            got = got[:nnz] if f in ("col_idx", "flag", "row_idx", "cflag") else got
+            assert np.array_equal(got, want[f]), f
+        assert int(bad.item()) == 0

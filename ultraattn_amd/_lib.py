@@ -14,6 +14,7 @@ _i32p, _u8p, _i64p = POINTER(c_int32), POINTER(c_uint8), POINTER(c_int64)
 SIGNATURES = {
     "ua_version": (c_int, []),
     "ua_strerror": (c_char_p, [c_int]),
+    "ua_init": (c_int, []),
     "ua_tilelist_size": (c_int, [c_void_p, c_int, c_int, c_int, _i64p, _i64p, _i64p]),
     "ua_tilelist_build": (c_int, [c_void_p, c_int, c_int, c_int] + [c_void_p] * 8),
     "ua_tilelist_build_device": (c_int, [c_void_p, c_int, c_int, c_int] + [c_void_p] * 10),
@@ -25,6 +26,8 @@ SIGNATURES = {
     "ua_merge": (c_int, [POINTER(c_void_p), POINTER(c_void_p), c_int, c_void_p, c_void_p,
                          c_int, c_int, c_int, c_int, c_void_p]),
     "ua_merge_update": (c_int, [c_void_p] * 6 + [c_int] * 7 + [_i64p] * 6 + [c_void_p]),
+    "ua_grad_accumulate": (c_int, [c_void_p, c_void_p, c_void_p, c_int64, c_int, c_void_p]),
+    "ua_grad_sum": (c_int, [POINTER(c_void_p), c_int, c_int, c_void_p, c_int, c_int, c_int, c_int, _i64p, c_float, c_void_p]),
     "ua_cols_gather": (c_int, [c_void_p, c_void_p, c_int, c_int, c_int64, c_void_p]),
     "ua_cols_scatter": (c_int, [c_void_p, c_void_p, c_int, c_int, c_int64, c_void_p]),
 }

@@ -9,7 +9,7 @@ PKG_DIR = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(PKG_DIR, "csrc")
 LIB_NAME = "libultraattn_hip.so"
 LIB_PATH = os.path.join(PKG_DIR, LIB_NAME)
-SOURCES = ["api.hip", "tilelist.hip", "merge.hip", "glue.hip", "fwd.hip", "bwd.hip"]
+SOURCES = ["api.hip", "tilelist.hip", "merge.hip", "glue.hip", "reduce.hip", "fwd.hip", "bwd.hip"]
 # benchmark-only probes (register-only MFMA loop, streaming-mix ceiling): built beside bench.py,
 # never linked into the product library
 BENCH_SRC = os.path.join(os.path.dirname(PKG_DIR), "bench_probe.hip")

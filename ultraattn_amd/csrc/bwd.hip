@@ -543,6 +543,7 @@ static int fill_common(BwdParams& p, const void* q, const void* k, const void* v
   if (!q || !k || !v || !dout || !lse || !delta || !qs || !ks || !vs || !ds) return UA_ERR_NULL;
   if (batch <= 0 || n_heads <= 0 || n_qtiles <= 0 || n_ktiles <= 0 || nnz < 0) return UA_ERR_SHAPE;
   if (nnz > 0 && (!idx || !flag)) return UA_ERR_NULL;          // only an empty list may leave them out
+  if (flag && !aligned4(flag)) return UA_ERR_ALIGN;            // read one aligned 32-bit word at a time
   if ((int64_t)batch * n_heads * n_qtiles > INT32_MAX || (int64_t)batch * n_heads * n_ktiles > INT32_MAX)
     return UA_ERR_SHAPE;
   if (head_dim != kHeadDim || !(softmax_scale > 0.f)) return UA_ERR_UNSUPPORTED;

@@ -237,6 +237,7 @@ extern "C" int ua_bsa_fwd(const void* q, const void* k, const void* v, void* o, 
     return UA_ERR_NULL;
   if (batch <= 0 || n_heads <= 0 || n_qtiles <= 0 || n_ktiles <= 0 || nnz < 0) return UA_ERR_SHAPE;
   if (nnz > 0 && (!col_idx || !flag)) return UA_ERR_NULL;      // only an empty list may leave them out
+  if (flag && !aligned4(flag)) return UA_ERR_ALIGN;            // read one aligned 32-bit word at a time
   if ((int64_t)batch * n_heads * n_qtiles > INT32_MAX) return UA_ERR_SHAPE;
   if (head_dim != kHeadDim || !(softmax_scale > 0.f)) return UA_ERR_UNSUPPORTED;
   if (!aligned16(q) || !aligned16(k) || !aligned16(v) || !aligned16(o)) return UA_ERR_ALIGN;

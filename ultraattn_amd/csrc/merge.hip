@@ -324,6 +324,11 @@ extern "C" int ua_merge_update(const void* out, const float* lse, const void* bl
   };
   if (!rows_ok(out, out_strides, out_is_fp32) || !rows_ok(block_out, block_out_strides, block_is_fp32) ||
       !rows_ok(new_out, new_out_strides, new_is_fp32)) return UA_ERR_ALIGN;
+  // in place (the slice_ path): same pointer means same element type and the same strides, else
+  // one thread's store would land on rows that other threads have not read yet
+  auto same3 = [](const int64_t* a, const int64_t* b) { return a[0] == b[0] && a[1] == b[1] && a[2] == b[2]; };
+  if (new_out == out && (out_is_fp32 != new_is_fp32 || !same3(out_strides, new_out_strides))) return UA_ERR_SHAPE;
+  if (new_lse == lse && !same3(lse_strides, new_lse_strides)) return UA_ERR_SHAPE;
   if (int rc = check_device()) return rc;
   UpdateParams p;
   p.out = out; p.lse = lse; p.blk = block_out; p.blk_lse = block_lse; p.new_out = new_out; p.new_lse = new_lse;

@@ -135,21 +135,27 @@ __global__ __launch_bounds__(64 * kWavesPerGroup) void tl_count_kernel(const uin
   if (lane == 0) (ln.is_row ? qcnt : kcnt)[ln.id] = n;
 }
 
-// check: a single workgroup counts the mask entries that are not a Block_Type (> 2); the
-// builder treats them as EMPTY, and the count lets the caller detect them after the stream
-// has been synchronised (the host builder returns UA_ERR_MASK for the same input).
-__global__ __launch_bounds__(1024) void tl_check_kernel(const uint8_t* mask, int64_t n, int32_t* n_invalid, int32_t* anchor_cnt) {
+// init: zeroes the counters that the later kernels of the stream accumulate into.
+__global__ void tl_init_kernel(int32_t* n_invalid, int32_t* anchor_cnt) {
+  if (threadIdx.x == 0) *n_invalid = 0;
+  if (threadIdx.x < 4) anchor_cnt[threadIdx.x] = 0;
+}
+
+// check: counts the mask entries that are not a Block_Type (> 2); the builder treats them as
+// EMPTY, and the count lets the caller detect them after the stream has been synchronised (the
+// host builder returns UA_ERR_MASK for the same input).  Grid-stride over the mask, one atomic per
+// workgroup.
+__global__ __launch_bounds__(1024) void tl_check_kernel(const uint8_t* mask, int64_t n, int32_t* n_invalid) {
   __shared__ int32_t part[16];
-  if (threadIdx.x < 4) anchor_cnt[threadIdx.x] = 0;      // counted by tl_anchor_kernel, later in the stream
   int bad = 0;
-  for (int64_t i = threadIdx.x; i < n; i += 1024) bad += mask[i] > 2;
+  for (int64_t i = (int64_t)blockIdx.x * 1024 + threadIdx.x; i < n; i += (int64_t)gridDim.x * 1024) bad += mask[i] > 2;
   bad = wave_sum(bad);
   if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = bad;
   __syncthreads();
   if (threadIdx.x == 0) {
     int s = 0;
     for (int i = 0; i < 16; ++i) s += part[i];
-    *n_invalid = s;
+    if (s) atomicAdd(n_invalid, s);
   }
 }
 
@@ -210,30 +216,47 @@ __global__ __launch_bounds__(64 * kWavesPerGroup) void tl_fill_kernel(const uint
 }
 
 // anchor: number of distinct first and of distinct last indices over the lines of each side that are
-// neither empty nor very long -> anchor_cnt[0..1] for the rows, [2..3] for the columns.  One workgroup
-// per line; the line counts if no earlier line of its side holds the same value.
-__global__ __launch_bounds__(256) void tl_anchor_kernel(const int32_t* qptr, const int32_t* qidx, int nq,
-                                                        const int32_t* kptr, const int32_t* kidx, int nk, int32_t* anchor_cnt) {
-  __shared__ int dup_s[2];
-  const int t = blockIdx.x;
-  const int32_t* ptr = t < nq ? qptr : kptr;
-  const int32_t* idx = t < nq ? qidx : kidx;
-  const int n = t < nq ? nq : nk;
-  const int i = t < nq ? t : t - nq;
+// neither empty nor very long -> anchor_cnt[0..1] for the rows, [2..3] for the columns.  Linear in
+// the number of lines: every line marks its two anchor values in a flag array indexed by tile id
+// (bit 0 = seen as a first index, bit 1 = as a last index), then the set bits are counted.  The flag
+// arrays are the launch-order outputs themselves, which are only written afterwards: a row's anchors
+// are key tiles (flags in k_order, n_ktiles entries), a column's are query tiles (flags in q_order).
+__global__ __launch_bounds__(256) void tl_anchor_clear_kernel(int32_t* q_order, int nq, int32_t* k_order, int nk) {
+  const int i = blockIdx.x * 256 + threadIdx.x;
+  if (i < nq) q_order[i] = 0;
+  else if (i < nq + nk) k_order[i - nq] = 0;
+}
+__global__ __launch_bounds__(256) void tl_anchor_mark_kernel(const int32_t* qptr, const int32_t* qidx, int nq,
+                                                             const int32_t* kptr, const int32_t* kidx, int nk,
+                                                             int32_t* q_order, int32_t* k_order) {
+  const int t = blockIdx.x * 256 + threadIdx.x;
+  if (t >= nq + nk) return;
+  const bool is_row = t < nq;
+  const int32_t* ptr = is_row ? qptr : kptr;
+  const int32_t* idx = is_row ? qidx : kidx;
+  const int n = is_row ? nq : nk, i = is_row ? t : t - nq;
   if (ptr[i + 1] == ptr[i] || very_long(ptr, n, i)) return;
-  if (threadIdx.x < 2) dup_s[threadIdx.x] = 0;
-  __syncthreads();
+  int32_t* flags = is_row ? k_order : q_order;
+  const int limit = is_row ? nk : nq;
   const int first = idx[ptr[i]], last = idx[ptr[i + 1] - 1];
-  bool df = false, dl = false;
-  for (int j = threadIdx.x; j < i; j += 256) {
-    if (ptr[j + 1] == ptr[j] || very_long(ptr, n, j)) continue;
-    df |= idx[ptr[j]] == first;
-    dl |= idx[ptr[j + 1] - 1] == last;
+  if (first >= 0 && first < limit) atomicOr(&flags[first], 1);
+  if (last >= 0 && last < limit) atomicOr(&flags[last], 2);
+}
+__global__ __launch_bounds__(256) void tl_anchor_count_kernel(const int32_t* q_order, int nq, const int32_t* k_order, int nk,
+                                                              int32_t* anchor_cnt) {
+  const int t = blockIdx.x * 256 + threadIdx.x;
+  // flags in k_order belong to the rows (anchor_cnt[0..1]), flags in q_order to the columns ([2..3])
+  const int f = t < nq ? q_order[t] : (t < nq + nk ? k_order[t - nq] : 0);
+  const bool rows_side = t >= nq;
+  // a wavefront may straddle the boundary between the two arrays: its two sides are summed separately
+  const int r0 = wave_sum(rows_side ? (f & 1) : 0), r1 = wave_sum(rows_side ? ((f >> 1) & 1) : 0);
+  const int c0 = wave_sum(rows_side ? 0 : (f & 1)), c1 = wave_sum(rows_side ? 0 : ((f >> 1) & 1));
+  if ((threadIdx.x & 63) == 0) {
+    if (r0) atomicAdd(&anchor_cnt[0], r0);
+    if (r1) atomicAdd(&anchor_cnt[1], r1);
+    if (c0) atomicAdd(&anchor_cnt[2], c0);
+    if (c1) atomicAdd(&anchor_cnt[3], c1);
   }
-  if (df) dup_s[0] = 1;
-  if (dl) dup_s[1] = 1;
-  __syncthreads();
-  if (threadIdx.x < 2 && !dup_s[threadIdx.x]) atomicAdd(&anchor_cnt[(t < nq ? 0 : 2) + threadIdx.x], 1);
 }
 
 // order: rank of a line = number of lines that precede it; one workgroup per line, its threads
@@ -330,16 +353,23 @@ static int build_device_impl(const uint8_t* block_mask, int n_qblocks, int n_kbl
   int32_t* qcnt = work;
   int32_t* kcnt = work + nqt + 1;
   int32_t* anchor_cnt = work + nqt + nkt + 3;
-  hipLaunchKernelGGL(tl_check_kernel, dim3(1), dim3(1024), 0, st, block_mask, (int64_t)n_qblocks * n_kblocks, n_invalid, anchor_cnt);
+  hipLaunchKernelGGL(tl_init_kernel, dim3(1), dim3(64), 0, st, n_invalid, anchor_cnt);
+  const int64_t n_mask = (int64_t)n_qblocks * n_kblocks;
+  hipLaunchKernelGGL(tl_check_kernel, dim3((unsigned)std::min<int64_t>((n_mask + 1023) / 1024, 2048)), dim3(1024), 0, st,
+                     block_mask, n_mask, n_invalid);
   const int blocks = (nqt + nkt + kWavesPerGroup - 1) / kWavesPerGroup;
   hipLaunchKernelGGL(tl_count_kernel, dim3(blocks), dim3(64 * kWavesPerGroup), 0, st, block_mask, n_qblocks, n_kblocks, rate, qcnt, kcnt);
   hipLaunchKernelGGL(tl_scan_kernel, dim3(1), dim3(1024), 0, st, (const int32_t*)qcnt, nqt, row_ptr);
   hipLaunchKernelGGL(tl_scan_kernel, dim3(1), dim3(1024), 0, st, (const int32_t*)kcnt, nkt, col_ptr);
   hipLaunchKernelGGL(tl_fill_kernel, dim3(blocks), dim3(64 * kWavesPerGroup), 0, st, block_mask, n_qblocks, n_kblocks, rate,
                      (const int32_t*)row_ptr, col_idx, flag, (const int32_t*)col_ptr, row_idx, cflag);
-  hipLaunchKernelGGL(tl_anchor_kernel, dim3(nqt + nkt), dim3(256), 0, st,
+  const int line_blocks = (nqt + nkt + 255) / 256;
+  hipLaunchKernelGGL(tl_anchor_clear_kernel, dim3(line_blocks), dim3(256), 0, st, q_order, nqt, k_order, nkt);
+  hipLaunchKernelGGL(tl_anchor_mark_kernel, dim3(line_blocks), dim3(256), 0, st,
                      (const int32_t*)row_ptr, (const int32_t*)col_idx, nqt,
-                     (const int32_t*)col_ptr, (const int32_t*)row_idx, nkt, anchor_cnt);
+                     (const int32_t*)col_ptr, (const int32_t*)row_idx, nkt, q_order, k_order);
+  hipLaunchKernelGGL(tl_anchor_count_kernel, dim3(line_blocks), dim3(256), 0, st,
+                     (const int32_t*)q_order, nqt, (const int32_t*)k_order, nkt, anchor_cnt);
   hipLaunchKernelGGL(tl_order_kernel, dim3(nqt + nkt), dim3(256), 0, st,
                      (const int32_t*)row_ptr, (const int32_t*)col_idx, nqt, q_order,
                      (const int32_t*)col_ptr, (const int32_t*)row_idx, nkt, k_order, rate, (const int32_t*)anchor_cnt);
@@ -387,6 +417,13 @@ static int scratch_of_current_device(int32_t** out) {
   }
   *out = p;
   return UA_OK;
+}
+
+// Everything the entry points resolve lazily per device, resolved now (outside any graph capture).
+extern "C" int ua_init(void) {
+  if (int rc = ua::check_device()) return rc;
+  int32_t* p = nullptr;
+  return scratch_of_current_device(&p);
 }
 
 extern "C" int ua_tilelist_build_device_noalloc(const uint8_t* block_mask, int n_qblocks, int n_kblocks, int rate,

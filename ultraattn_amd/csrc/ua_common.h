@@ -93,7 +93,8 @@ __device__ __forceinline__ int32_t sload(const int32_t* p, int i) {
   return ((const __attribute__((address_space(4))) int32_t*)p)[i];
 }
 __device__ __forceinline__ int sload(const uint8_t* p, int i) {
-  // the scalar unit loads dwords: fetch the aligned word that holds byte i
+  // the scalar unit loads dwords: fetch the aligned word that holds byte i (the entry points
+  // require p on a 4-byte boundary and the array padded to a multiple of 4 bytes)
   const uintptr_t a = reinterpret_cast<uintptr_t>(p) + (uintptr_t)i;
   const uint32_t w = *reinterpret_cast<const __attribute__((address_space(4))) uint32_t*>(a & ~(uintptr_t)3);
   return (w >> (8 * (a & 3))) & 0xff;
@@ -163,6 +164,7 @@ __device__ __forceinline__ void map_block(int bid, int nbh, int heads_per_xcd, i
   }
 }
 
+inline bool aligned4(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 3) == 0; }
 inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
 inline bool strides_ok(const int64_t* s) { return s && s[0] % 8 == 0 && s[1] % 8 == 0 && s[2] % 8 == 0 && s[1] > 0; }
 

@@ -16,7 +16,7 @@ import numpy as np
 import torch
 
 from .masks import CAUSAL, EMPTY, FULL
-from .ops import bsa_bwd, bsa_fwd, merge_partials, softmax_delta
+from .ops import bsa_bwd, bsa_fwd, grad_sum, merge_partials, softmax_delta
 from .tilelist import TileList, build_tile_list
 
 Ids = Union[int, Tuple[int, ...]]
@@ -82,6 +82,7 @@ class BlockSparseExecutor:
         self.softmax_scale = softmax_scale
         self.tiles: TileList = build_tile_list(self.mask, block=self.chunk)
         self.kernel_tiles: List[TileList] = []
+        self._parts, self._part_key = None, None
         if kernel_tiles > 1:
             cols = np.nonzero(self.mask.any(0))[0]
             for part in np.array_split(cols, min(kernel_tiles, max(1, len(cols)))):
@@ -103,11 +104,25 @@ class BlockSparseExecutor:
         st = st.reshape(st.shape[-2:])
         return cls(np.where(st == rank, np.asarray(block_table, np.uint8), EMPTY).astype(np.uint8), chunk, **kw)
 
+    def _partials(self, q):
+        """The partial (O, LSE) buffers of the kernel tiles, allocated on the first call for a shape
+        and device and reused afterwards (a serving loop then allocates nothing per step)."""
+        key = (tuple(q.shape), q.device)
+        if self._part_key != key:
+            B, Sq, Nh, _ = q.shape
+            self._parts = [(torch.empty(q.shape, dtype=q.dtype, device=q.device),
+                            torch.empty(B, Nh, Sq, dtype=torch.float32, device=q.device)) for _ in self.kernel_tiles]
+            self._part_key = key
+        return self._parts
+
     def forward(self, q, k, v, out=None, lse=None):
-        """-> (out, lse); one launch, or ``kernel_tiles`` launches + one merge."""
+        """-> (out, lse); one launch, or ``kernel_tiles`` launches into partial buffers that the
+        executor keeps + one merge.  The partials are overwritten by the next call with kernel
+        tiles, so calls on different streams must not overlap."""
         if not self.kernel_tiles:
             return bsa_fwd(q, k, v, self.tiles, self.softmax_scale, out=out, lse=lse)
-        parts = [bsa_fwd(q, k, v, t, self.softmax_scale) for t in self.kernel_tiles]
+        parts = [bsa_fwd(q, k, v, t, self.softmax_scale, out=po, lse=pl)
+                 for t, (po, pl) in zip(self.kernel_tiles, self._partials(q))]
         return merge_partials([p[0] for p in parts], [p[1] for p in parts], out=out, lse=lse)
 
     def backward(self, dout, q, k, v, out, lse, dq=None, dk=None, dv=None, softmax_d=None):
@@ -126,8 +141,6 @@ class BlockSparseExecutor:
     @staticmethod
     def reduce_bwd(parts: Sequence[torch.Tensor]) -> torch.Tensor:
         """``Output_Row_Bwd.reduce`` / ``Output_Col_Bwd.reduce``: fp32 sum of partial gradients
-        (``ring_flash_attn/ring_flash_attn.py:110-118`` accumulates in fp32), returned in bf16."""
-        acc = parts[0].float()
-        for p in parts[1:]:
-            acc += p.float()
-        return acc.to(parts[0].dtype)
+        (``ring_flash_attn/ring_flash_attn.py:110-118`` accumulates in fp32), returned in bf16; one
+        pass over up to 16 partials (``ua_grad_sum``)."""
+        return grad_sum([p if p.is_contiguous() else p.contiguous() for p in parts])

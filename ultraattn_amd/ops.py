@@ -187,6 +187,59 @@ def merge_partials(outs: Sequence[torch.Tensor], lses: Sequence[torch.Tensor],
     return out, lse
 
 
+def grad_accumulate(partial: torch.Tensor, out: Optional[torch.Tensor], acc: Optional[torch.Tensor] = None,
+                    init_from_out: bool = False) -> None:
+    """One step of the gradient accumulation that the reference specifies
+    (``ring_flash_attn/ring_flash_attn.py:110-118``) and its packs leave as stubs
+    (``orchestrated_attn/utils.py:260-262, 296-298``), as one kernel (``ua_grad_accumulate``):
+
+    * ``acc`` (fp32) given: ``acc += partial`` and ``out = bf16(acc)`` (``out`` may be None);
+      with ``init_from_out`` the sum starts from ``out``: ``acc = float(out) + partial``;
+    * no ``acc``: ``out = bf16(float(out) + partial)``.
+    ``partial`` and ``out`` are contiguous bf16 tensors of equal size, ``acc`` contiguous fp32."""
+    n = partial.numel()
+    for name, t, dt in (("partial", partial, torch.bfloat16), ("out", out, torch.bfloat16), ("acc", acc, torch.float32)):
+        if t is None:
+            continue
+        if not t.is_cuda or t.dtype != dt or not t.is_contiguous() or t.numel() != n:
+            raise ValueError(f"{name} must be a contiguous {dt} CUDA tensor of {n} elements")
+    lib = _lib.load()
+    with torch.cuda.device(partial.device):
+        st = torch.cuda.current_stream().cuda_stream
+        rc = lib.ua_grad_accumulate(acc.data_ptr() if acc is not None else None, partial.data_ptr(),
+                                    out.data_ptr() if out is not None else None, n, int(init_from_out), st)
+    _lib.check(rc, "ua_grad_accumulate")
+
+
+def grad_sum(parts: Sequence[torch.Tensor], out: Optional[torch.Tensor] = None, scale: float = 1.0) -> torch.Tensor:
+    """``out = bf16(scale * sum(parts))`` with the sum carried in fp32, one pass (``ua_grad_sum``).
+    parts: 1..16 contiguous ``[B, S, Nh, 128]`` tensors, all bf16 or all fp32; ``out`` bf16, may be a
+    strided view (head_dim contiguous)."""
+    if not parts:
+        raise ValueError("need at least one partial gradient")
+    dt = parts[0].dtype
+    if dt not in (torch.bfloat16, torch.float32):
+        raise TypeError("partial gradients must be bfloat16 or float32")
+    for t in parts:
+        if not t.is_cuda or t.dtype != dt or t.shape != parts[0].shape or not t.is_contiguous() or t.dim() != 4 \
+                or t.shape[-1] != HEAD_DIM:
+            raise ValueError("partial gradients must be contiguous [B, S, Nh, 128] CUDA tensors of one dtype and shape")
+    B, S, Nh, D = parts[0].shape
+    if out is None:
+        out = torch.empty(parts[0].shape, dtype=torch.bfloat16, device=parts[0].device)
+    _check_qkv("out", out, 1)
+    if out.shape != parts[0].shape:
+        raise ValueError("out must have the partials' shape")
+    pp = (ctypes.c_void_p * len(parts))(*[t.data_ptr() for t in parts])
+    lib = _lib.load()
+    with torch.cuda.device(out.device):
+        st = torch.cuda.current_stream().cuda_stream
+        rc = lib.ua_grad_sum(pp, len(parts), int(dt == torch.float32), out.data_ptr(), B, S, Nh, D,
+                             _lib.strides3(out), float(scale), st)
+    _lib.check(rc, "ua_grad_sum")
+    return out
+
+
 def _strides_bsh(t: torch.Tensor, layout: str):
     """(batch, token, head) element strides of a statistics tensor given as [B, S, Nh, 1]
     ('bsh1') or [B, Nh, S] ('bhs'), or of a [B, S, Nh, D] row tensor ('rows')."""
@@ -239,6 +292,11 @@ def update_out_and_lse(out: Optional[torch.Tensor], lse: Optional[torch.Tensor],
     _check_rows("block_out", block_out)
     if slice_ is not None:
         tgt_out, tgt_lse = out[slice_], lse[slice_]
+        if tgt_out.untyped_storage().data_ptr() != out.untyped_storage().data_ptr() or \
+                tgt_lse.untyped_storage().data_ptr() != lse.untyped_storage().data_ptr():
+            # the reference assigns `out[slice_] = ...`, which writes through any index; a kernel can
+            # only write through a view
+            raise ValueError("slice_ must select a view of out and lse (slices, not index lists or tensors)")
         new_out, new_lse = tgt_out, tgt_lse                    # views: written in place
     else:
         tgt_out, tgt_lse = out, lse

@@ -9,7 +9,7 @@ Backward: row in  = [Q | dO | D (fp32) | lse]          col in = [K | V]
           row out = [dQ]                               col out = [dK | dV]
 """
 import math
-from typing import Tuple
+from typing import Iterable, Optional, Tuple
 
 import torch
 
@@ -62,12 +62,35 @@ class OutputRowFwd:
     def __init__(self, buf: torch.Tensor, q_shape: Tuple[int, int, int, int], lse: torch.Tensor = None):
         self.data = _take(buf, 0, math.prod(q_shape))
         self.O = self.data.view(q_shape)
-        B, S, Nh, _ = q_shape
-        self.lse = lse if lse is not None else torch.full((B, Nh, S), float("-inf"), dtype=FULL_DTYPE, device=buf.device)
+        self._lse = lse
+
+    @property
+    def lse(self) -> torch.Tensor:
+        """fp32 [B, Nh, S]; allocated (as "no keys seen", -inf) on first use when none was given."""
+        if self._lse is None:
+            B, S, Nh, _ = self.O.shape
+            self._lse = torch.full((B, Nh, S), float("-inf"), dtype=FULL_DTYPE, device=self.data.device)
+        return self._lse
+
+    @lse.setter
+    def lse(self, value: torch.Tensor) -> None:
+        self._lse = value
 
     def reduce(self, other: "OutputRowFwd") -> None:
         from .ops import merge_partials
         merge_partials([self.O, other.O], [self.lse, other.lse], out=self.O, lse=self.lse)
+
+
+class OutputColFwd:
+    """``Output_Col_Fwd`` (``orchestrated_attn/utils.py:137-146``): the forward produces nothing
+    per column; the class exists so that the buffer dictionary has all four corners."""
+
+    def __init__(self, buf: torch.Tensor = None, k_shape=None):
+        self.data = None
+
+    @staticmethod
+    def numel(k_shape) -> int:
+        return 0
 
 
 class InputRowBwd:
@@ -105,18 +128,40 @@ class InputRowBwd:
 
 
 class _Fp32Accumulated:
-    """``reduce`` for gradient packs: the running sum is kept in fp32 beside the bf16 pack (the
-    accumulation the reference specifies, ``ring_flash_attn/ring_flash_attn.py:110-118``: partial
-    gradients are added into fp32 buffers and cast once), and ``data`` always holds its bf16
-    rounding.  Summing in bf16 instead loses about half a bit per partial."""
+    """``reduce`` for gradient packs, the accumulation the reference specifies
+    (``ring_flash_attn/ring_flash_attn.py:110-118``: partial gradients are added into fp32 buffers
+    and cast once) and leaves commented out in its packs.
+
+    The pack is a view into a persistent buffer that kernels and receives rewrite in place, so no
+    fp32 state outlives a reduction chain: ``begin_reduce()`` opens one (the running sum then
+    lives in fp32, in ``acc`` when the caller supplies the buffer), every ``reduce(other)`` adds
+    one partial and leaves the bf16 rounding of the sum in ``data``, ``end_reduce()`` drops the
+    fp32 sum.  Outside a chain ``reduce`` is stateless: ``data = bf16(float(data) + other)``,
+    which costs about half a bit per partial but can never mix in a stale sum."""
     data: torch.Tensor
     _acc = None
+    _acc_live = False
+
+    def begin_reduce(self, acc: torch.Tensor = None) -> None:
+        n = self.data.numel()
+        if acc is None:
+            acc = torch.empty(n, dtype=FULL_DTYPE, device=self.data.device)
+        if acc.dtype != FULL_DTYPE or acc.numel() < n or not acc.is_contiguous() or acc.device != self.data.device:
+            raise ValueError(f"acc must be a contiguous float32 tensor of at least {n} elements on the pack's device")
+        self._acc = acc.view(-1)[:n]
+        self._acc_live = False            # the first reduce() initialises it from data
+
+    def end_reduce(self) -> None:
+        self._acc = None
+        self._acc_live = False
 
     def reduce(self, other) -> None:
+        from .ops import grad_accumulate
         if self._acc is None:
-            self._acc = self.data.to(FULL_DTYPE)
-        self._acc.add_(other.data)            # bf16 -> fp32 promotion happens inside the add
-        self.data.copy_(self._acc)
+            grad_accumulate(other.data, self.data)
+        else:
+            grad_accumulate(other.data, self.data, acc=self._acc, init_from_out=not self._acc_live)
+            self._acc_live = True
 
 
 class OutputRowBwd(_Fp32Accumulated):
@@ -176,3 +221,90 @@ def scatter_cols(col_out: OutputColBwd, n_chunks: int, k_shape, out: torch.Tenso
     (``oc.view(2, Y, K_nelem).transpose(0,1).contiguous()``,
     ``orchestrated_attn/orchestrated_attn_impl.py:548``)."""
     return _permute_cols("ua_cols_scatter", col_out.data, n_chunks, k_shape, out)
+
+
+def _scaled(shape: Tuple[int, int, int, int], n_chunks: int) -> Tuple[int, int, int, int]:
+    """Shape of ``n_chunks`` partitions side by side (``get_Q_shape_from_da_config`` /
+    ``get_K_shape_from_da_config``, ``orchestrated_attn/utils.py:25-29``)."""
+    return (shape[0], shape[1] * n_chunks, shape[2], shape[3])
+
+
+def create_buf_dict(q_shape, k_shape, fob: int, tensor_buf: torch.Tensor, comp_keys: Iterable = (),
+                    fused_xy: Optional[Tuple[int, int]] = None, level_rank: int = 0,
+                    batch_degrees: Tuple[int, int] = (1, 1), lse_slots: int = 1) -> dict:
+    """Carves the packs of one execution plan out of ``tensor_buf`` (flat bf16), with the keys and
+    offsets of the reference's ``create_buf_dict`` (``search_algo/benchmark.py:231-334``).
+
+    ``q_shape`` / ``k_shape``: ``(bs, S_per_partition, Nh, D)`` of one row / column partition;
+    ``fob`` 0 forward, 1 backward; ``batch_degrees`` the (row, column) partitions per kernel of
+    the level above.
+
+    General graph (``fused_xy=None``): ``(('i'|'o', 'r'|'c'), n) -> pack`` over ``n`` partitions
+    for ``n = 1`` and for every ``low_bds`` that the ``Comp_Kernel`` keys ``(b, h, rid, cid, gpu)``
+    in ``comp_keys`` need (ids may be tuples, the fused rectangles of
+    ``search_algo/graph_transformation_engine.py:83``); as in the reference every pack starts at
+    offset 0 of the same buffer (``:254-283``: the harness times kernels, the addresses are
+    dummies), plus ``graph_type``, ``tensor_buf``, ``inp_row``, ``inp_col``, ``out_row``, ``out_col``.
+
+    Fused X x Y graph (``fused_xy=(X, Y)``): the flat slices ``ir | ic | or | oc`` with
+    ``ir_nelems = bs*Sq*Nh*D`` (forward) or ``bs*Sq*Nh*(2D + 2 + lse_slots)`` (backward: Q, dO, D, lse),
+    ``ic_nelems = bs*Skv*Nh*2D``, ``or_nelems = bs*Sq*Nh*D``, ``oc_nelems = 0 | bs*Skv*Nh*2D``, the
+    totals ``*_tot = *_nelems * X`` (rows) or ``* Y`` (columns), for the backward the second row
+    buffer (``ir`` = the extra one, ``ir_`` = the first, ``:318-323``), and ``inp_row`` / ``inp_col`` =
+    this rank's pack inside ``ir`` / ``ic`` (x = rank % X, y = rank // X, ``:326-329``).
+
+    ``lse_slots=1`` is the reference's footprint (its ``lse`` view is bf16, an artefact of a harness
+    that never reads it back); ``lse_slots=2`` keeps a usable fp32 ``lse`` in every backward row pack."""
+    if fob not in (0, 1):
+        raise ValueError("fob must be 0 (forward) or 1 (backward)")
+    if len(batch_degrees) != 2:
+        raise ValueError(f"Invalid batch_degrees: {batch_degrees}")
+    bs, Sq, Nh, D = q_shape
+    Skv = k_shape[1]
+    row_in = (lambda buf, n: InputRowFwd(buf, _scaled(q_shape, n))) if fob == 0 else \
+        (lambda buf, n: InputRowBwd(buf, _scaled(q_shape, n), lse_slots=lse_slots))
+    col_in = lambda buf, n: InputColFwd(buf, _scaled(k_shape, n))
+    row_out = (lambda buf, n: OutputRowFwd(buf, _scaled(q_shape, n))) if fob == 0 else \
+        (lambda buf, n: OutputRowBwd(buf, _scaled(q_shape, n)))
+    col_out = (lambda buf, n: OutputColFwd()) if fob == 0 else (lambda buf, n: OutputColBwd(buf, _scaled(k_shape, n)))
+    if fused_xy is None:
+        d = {}
+
+        def add_rows(n):
+            if (("i", "r"), n) not in d:
+                d[(("i", "r"), n)] = row_in(tensor_buf, batch_degrees[0] * n)
+                d[(("o", "r"), n)] = row_out(tensor_buf, batch_degrees[0] * n)
+
+        def add_cols(n):
+            if (("i", "c"), n) not in d:
+                d[(("i", "c"), n)] = col_in(tensor_buf, batch_degrees[1] * n)
+                d[(("o", "c"), n)] = col_out(tensor_buf, batch_degrees[1] * n)
+        add_rows(1)
+        add_cols(1)
+        for key in comp_keys:
+            rid, cid = key[2], key[3]
+            add_rows(len(rid) if isinstance(rid, tuple) else 1)
+            add_cols(len(cid) if isinstance(cid, tuple) else 1)
+        d.update(graph_type="general", tensor_buf=tensor_buf, inp_row=d[(("i", "r"), 1)], inp_col=d[(("i", "c"), 1)],
+                 out_row=d[(("o", "r"), 1)], out_col=d[(("o", "c"), 1)])
+        return d
+    X, Y = fused_xy
+    sq, skv = Sq * batch_degrees[0], Skv * batch_degrees[1]
+    ir_nelems = bs * sq * Nh * (D if fob == 0 else 2 * D + 2 + lse_slots)
+    ic_nelems = bs * skv * Nh * 2 * D
+    or_nelems = bs * sq * Nh * D
+    oc_nelems = 0 if fob == 0 else bs * skv * Nh * 2 * D
+    ir_tot, ic_tot, or_tot, oc_tot = ir_nelems * X, ic_nelems * Y, or_nelems * X, oc_nelems * Y
+    end = ir_tot + ic_tot + or_tot + oc_tot
+    buf = _take(tensor_buf, 0, end + (ir_tot if fob == 1 else 0))
+    d = {"ir": buf[:ir_tot], "ic": buf[ir_tot:ir_tot + ic_tot], "or": buf[ir_tot + ic_tot:ir_tot + ic_tot + or_tot],
+         "oc": buf[ir_tot + ic_tot + or_tot:end],
+         "ir_nelems": ir_nelems, "ic_nelems": ic_nelems, "or_nelems": or_nelems, "oc_nelems": oc_nelems,
+         "ir_tot": ir_tot, "ic_tot": ic_tot, "or_tot": or_tot, "oc_tot": oc_tot, "graph_type": "fused"}
+    if fob == 1:
+        d["ir_"] = d["ir"]
+        d["ir"] = buf[end:end + ir_tot]
+    x, y = level_rank % X, level_rank // X
+    d["inp_row"] = row_in(d["ir"][ir_nelems * x:ir_nelems * (x + 1)], batch_degrees[0])
+    d["inp_col"] = col_in(d["ic"][ic_nelems * y:ic_nelems * (y + 1)], batch_degrees[1])
+    return d

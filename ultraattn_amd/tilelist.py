@@ -52,9 +52,32 @@ class TileList:
         import torch
         key = str(torch.device(device))
         if key not in self._dev:
-            self._dev[key] = {n: torch.from_numpy(np.ascontiguousarray(getattr(self, n))).to(device)
-                              for n in _HOST_FIELDS}
-        return self._dev[key]
+            # staged through pinned host memory and copied on the current stream without a host
+            # synchronisation; the flag arrays are padded to a multiple of 4 bytes (the kernels read
+            # them one aligned 32-bit word at a time)
+            dev, pinned = {}, []
+            for n in _HOST_FIELDS:
+                a = np.ascontiguousarray(getattr(self, n))
+                size = -(-max(a.shape[0], 1) // 4) * 4
+                host = torch.zeros(size, dtype=torch.from_numpy(a).dtype, pin_memory=True)
+                host[:a.shape[0]].copy_(torch.from_numpy(a))
+                full = host.to(device, non_blocking=True)
+                dev[n] = full[:a.shape[0]] if a.shape[0] else full[:0]
+                pinned.append(host)
+            dev["_pinned"] = pinned         # kept alive: the copies may still be in flight
+            dev["_ready"] = torch.cuda.Event()
+            dev["_ready"].record()
+            self._dev[key] = dev
+            return dev
+        dev = self._dev[key]
+        ready = dev.get("_ready")
+        if ready is not None:
+            if ready.query():
+                dev["_ready"] = None
+                dev["_pinned"] = None
+            else:                           # a later use on another stream orders itself behind the copies
+                torch.cuda.current_stream().wait_event(ready)
+        return dev
 
 
 def build_tile_list(block_mask, block: int = 512, tile: int = TILE, causal: bool = False,
@@ -105,7 +128,7 @@ def build_tile_list_device(block_mask_dev, block: int = 512, nnz: Optional[int] 
     nqb, nkb = m.shape
     nqt, nkt = nqb * rate, nkb * rate
     cap = nnz if nnz is not None else nqt * nkt
-    alloc = max(cap, 1)          # keep the pointers non-NULL for an empty list
+    alloc = -(-max(cap, 1) // 4) * 4   # non-NULL for an empty list; flag arrays padded to whole 32-bit words
     dev = m.device
     i32 = dict(dtype=torch.int32, device=dev)
     u8 = dict(dtype=torch.uint8, device=dev)
