@@ -160,6 +160,37 @@ int ua_bsa_bwd_dq(const void *q, const void *k, const void *v, const void *dout,
                   const int64_t *do_strides, const int64_t *dq_strides,
                   float softmax_scale, void *stream);
 
+/* ---- dense rectangles: the reference's tile kernel itself ------------------------------------
+ * One call = one `_flash_attn_forward(q, k, v, dropout_p=0, softmax_scale, causal, ..., out=)`
+ * (orchestrated_attn/orchestrated_attn_impl.py:326-337, hierarchy_attn/hierarchy_attn_impl.py:41-51)
+ * or one `_flash_attn_backward(dout, q, k, v, out, softmax_lse, dq, dk, dv, ..., softmax_d=)`
+ * (orchestrated_attn_impl.py:578-596) over a dense seqlen_q x seqlen_k rectangle (multiples of 128),
+ * with no tile list: the kernels enumerate the tiles themselves.  causal != 0 aligns the diagonal
+ * to the bottom-right corner as flash-attn >= 2.1 does (query i sees key j iff
+ * j <= i + seqlen_k - seqlen_q; rows that see no key get o = 0, lse = -inf, zero gradients).
+ * Rectangles with few tile lines (B * Nh * seqlen / 128 well below two workgroups per CU) and long
+ * walks are cut into up to UA_MAX_PARTS parts that run as workgroups of their own: the forward
+ * leaves partial (O, LSE) and finishes with ua_merge's kernel, the backward leaves fp32 partial
+ * dQ (parts of the key range) and dK, dV (parts of the query range) and sums them in one pass.
+ * The partials live in `workspace` (device memory, 16-byte aligned, caller-owned, overwritten by
+ * every call: calls that share it must not overlap); ua_dense_workspace_bytes() gives the size
+ * that lets a shape split (0 = it never splits).  With workspace == NULL or too small, or a
+ * forward output that is not contiguous, the call runs unsplit: same results, one workgroup per
+ * line.                                                                                       */
+int64_t ua_dense_workspace_bytes(int batch, int n_heads, int seqlen_q, int seqlen_k, int backward);
+int ua_dense_fwd(const void *q, const void *k, const void *v, void *o, float *lse,
+                 int batch, int n_heads, int seqlen_q, int seqlen_k, int head_dim,
+                 const int64_t *q_strides, const int64_t *k_strides, const int64_t *v_strides,
+                 const int64_t *o_strides, float softmax_scale, int causal,
+                 void *workspace, int64_t workspace_bytes, void *stream);
+int ua_dense_bwd(const void *dout, const void *q, const void *k, const void *v,
+                 const float *lse, const float *delta, void *dq, void *dk, void *dv,
+                 int batch, int n_heads, int seqlen_q, int seqlen_k, int head_dim,
+                 const int64_t *q_strides, const int64_t *k_strides, const int64_t *v_strides,
+                 const int64_t *do_strides, const int64_t *dq_strides, const int64_t *dk_strides,
+                 const int64_t *dv_strides, float softmax_scale, int causal,
+                 void *workspace, int64_t workspace_bytes, void *stream);
+
 /* ---- merge of partial outputs ---------------------------------------------------------------
  * Replaces the chain of `update_out_and_lse` calls (ring_flash_attn/utils.py:38-52, 78-99;
  * hierarchy_attn/utils.py:16-56; the commented formula at orchestrated_attn/utils.py:120-133)

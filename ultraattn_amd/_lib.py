@@ -23,6 +23,9 @@ SIGNATURES = {
     "ua_bsa_bwd_delta": (c_int, [c_void_p] * 3 + [c_int] * 4 + [_i64p] * 2 + [c_void_p]),
     "ua_bsa_bwd_dkdv": (c_int, [c_void_p] * 12 + [c_int] * 6 + [_i64p] * 6 + [c_float, c_void_p]),
     "ua_bsa_bwd_dq": (c_int, [c_void_p] * 11 + [c_int] * 6 + [_i64p] * 5 + [c_float, c_void_p]),
+    "ua_dense_workspace_bytes": (c_int64, [c_int] * 5),
+    "ua_dense_fwd": (c_int, [c_void_p] * 5 + [c_int] * 5 + [_i64p] * 4 + [c_float, c_int, c_void_p, c_int64, c_void_p]),
+    "ua_dense_bwd": (c_int, [c_void_p] * 9 + [c_int] * 5 + [_i64p] * 7 + [c_float, c_int, c_void_p, c_int64, c_void_p]),
     "ua_merge": (c_int, [POINTER(c_void_p), POINTER(c_void_p), c_int, c_void_p, c_void_p,
                          c_int, c_int, c_int, c_int, c_void_p]),
     "ua_merge_update": (c_int, [c_void_p] * 6 + [c_int] * 7 + [_i64p] * 6 + [c_void_p]),

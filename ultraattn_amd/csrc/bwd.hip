@@ -30,6 +30,13 @@ struct BwdParams {
   Strides3 qs, ks, vs, ds, o0s, o1s;
   float scale_log2, scale;
   int heads_per_xcd;
+  // Dense rectangle (no list arrays).  dq walks key tiles [0, n_ktiles) of a query tile, with
+  // dense_causal [0, qt + diag_off], the last one causal; dkdv walks query tiles [0, n_qtiles) of a
+  // key tile, with dense_causal [kt - diag_off, n_qtiles), the first one causal.  The walk is cut
+  // into n_parts parts of part_len tiles; with out_f32 part i leaves an fp32 partial result at
+  // out + i * o*_part (fp32 elements, contiguous [batch, tokens, heads, 128]) for a later sum.
+  int dense, dense_causal, diag_off, n_parts, part_len, out_f32;
+  int64_t o0_part, o1_part;
 };
 
 __device__ __forceinline__ void store_acc_t(bf16* row_ptr, const f32x16 (&acc)[4], float mul, int hi) {
@@ -43,6 +50,25 @@ __device__ __forceinline__ void store_acc_t(bf16* row_ptr, const f32x16 (&acc)[4
       for (int j = 0; j < 4; ++j) w[j] = (bf16)(acc[mb][4 * g + j] * mul);
       *reinterpret_cast<bf16x4*>(row_ptr + 32 * mb + 8 * g + 4 * hi) = w;
     }
+}
+
+__device__ __forceinline__ void store_acc_f32(float* row_ptr, const f32x16 (&acc)[4], float mul, int hi) {
+#pragma unroll
+  for (int mb = 0; mb < 4; ++mb)
+#pragma unroll
+    for (int g = 0; g < 4; ++g)
+      *reinterpret_cast<f32x4*>(row_ptr + 32 * mb + 8 * g + 4 * hi) =
+          f32x4{acc[mb][4 * g] * mul, acc[mb][4 * g + 1] * mul, acc[mb][4 * g + 2] * mul, acc[mb][4 * g + 3] * mul};
+}
+// Output row of a result tensor: the caller's strided bf16 tensor, or part `part` of the fp32 partials.
+__device__ __forceinline__ void store_result(const BwdParams& p, bf16* out, const Strides3& os, int64_t part_stride, int part,
+                                             int b, int64_t row, int h, int64_t seq, const f32x16 (&acc)[4], float mul, int hi) {
+  if (p.out_f32) {
+    float* base = reinterpret_cast<float*>(out) + part * part_stride;
+    store_acc_f32(base + (((int64_t)b * seq + row) * p.n_heads + h) * kHeadDim, acc, mul, hi);
+  } else {
+    store_acc_t(out + b * os.b + row * os.s + h * os.h, acc, mul, hi);
+  }
 }
 
 constexpr int kHalf = 64;
@@ -214,7 +240,7 @@ __device__ __forceinline__ void dkdv_ds_from_p(const u32x4 (&praw)[2], const f32
 // same sequence of barriers.
 template <bool kGroupB>
 __device__ __forceinline__ void dkdv_run(const BwdParams& p, uint32_t lds_base, int kt, int b,
-                                         int h, int tid, int lane, int wave8) {
+                                         int h, int tid, int lane, int wave8, int e0, int e1, int diag, int part) {
   const int wave = wave8 & 3, l32 = lane & 31, hi = lane >> 5;
   const int64_t seq_q = (int64_t)p.n_qtiles * kTile;
   // group A keeps the K fragments, group B the V fragments (B operands): lane holds key row
@@ -264,7 +290,6 @@ __device__ __forceinline__ void dkdv_run(const BwdParams& p, uint32_t lds_base, 
   const int q_half = kHalf * q_stride * 2, do_half = kHalf * do_stride * 2;
   const uint32_t q_extent = (uint32_t)((kTile - 1) * q_stride + kHeadDim) * 2;
   const uint32_t do_extent = (uint32_t)((kTile - 1) * do_stride + kHeadDim) * 2;
-  const int e0 = min(max(sload(p.ptr, kt), 0), p.nnz), e1 = min(max(sload(p.ptr, kt + 1), e0), p.nnz);
   const int n_half = 2 * (e1 - e0);
   // half tile i = half (i & 1) of list entry e0 + i / 2.  The list entry (query tile, causal
   // flag) of half tile i+1 is fetched one step before it is needed, so that no step starts by
@@ -272,6 +297,7 @@ __device__ __forceinline__ void dkdv_run(const BwdParams& p, uint32_t lds_base, 
   auto entry = [&](int i) {           // query tile | causal flag << 30
     if (n_half == 0) return 0;        // an empty column owns no list entry (the arrays may be NULL)
     const int e = min(e0 + (i >> 1), e1 - 1);
+    if (p.dense) return e | ((int)(e == diag) << 30);      // the entry is the query tile itself
     return min(max(sload(p.idx, e), 0), p.n_qtiles - 1) | (sload(p.flag, e) << 30);
   };
   // rows' statistics, staged in the form the accumulators start from: threads 0..63 carry
@@ -382,8 +408,9 @@ __device__ __forceinline__ void dkdv_run(const BwdParams& p, uint32_t lds_base, 
     step(i + 1, std::integral_constant<int, 1>{});
     step(i + 2, std::integral_constant<int, 2>{});
   }
-  if (kGroupB) store_acc_t(p.out0 + b * p.o0s.b + (int64_t)krow * p.o0s.s + h * p.o0s.h, acc, p.scale, hi);
-  else         store_acc_t(p.out1 + b * p.o1s.b + (int64_t)krow * p.o1s.s + h * p.o1s.h, acc, 1.f, hi);
+  const int64_t seq_k = (int64_t)p.n_ktiles * kTile;
+  if (kGroupB) store_result(p, p.out0, p.o0s, p.o0_part, part, b, krow, h, seq_k, acc, p.scale, hi);
+  else         store_result(p, p.out1, p.o1s, p.o1_part, part, b, krow, h, seq_k, acc, 1.f, hi);
 }
 
 __global__ __launch_bounds__(512) void dkdv_kernel(const BwdParams p) {
@@ -392,11 +419,23 @@ __global__ __launch_bounds__(512) void dkdv_kernel(const BwdParams p) {
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave8 = __builtin_amdgcn_readfirstlane(tid >> 6);      // 0..7
   int pos, bh;
-  map_block(blockIdx.x, p.batch * p.n_heads, p.heads_per_xcd, p.n_ktiles, pos, bh);
-  const int kt = min(max(sload(p.order, pos), 0), p.n_ktiles - 1);
+  map_block(blockIdx.x, p.batch * p.n_heads, p.heads_per_xcd, p.n_ktiles * p.n_parts, pos, bh);
   const int b = bh / p.n_heads, h = bh % p.n_heads;
-  if (wave8 >= 4) dkdv_run<true>(p, lds_base, kt, b, h, tid, lane, wave8);
-  else            dkdv_run<false>(p, lds_base, kt, b, h, tid, lane, wave8);
+  int kt, e0, e1, diag = -1, part = 0;
+  if (p.dense) {
+    part = pos / p.n_ktiles;
+    kt = pos - part * p.n_ktiles;                          // column 0 is the longest of a causal rectangle
+    if (p.dense_causal) diag = kt - p.diag_off;            // query tile on the diagonal (may lie outside)
+    const int qbeg = p.dense_causal ? min(max(diag, 0), p.n_qtiles) : 0;
+    e0 = min(max(part * p.part_len, qbeg), p.n_qtiles);
+    e1 = max(min((part + 1) * p.part_len, p.n_qtiles), e0);
+  } else {
+    kt = min(max(sload(p.order, pos), 0), p.n_ktiles - 1);
+    e0 = min(max(sload(p.ptr, kt), 0), p.nnz);
+    e1 = min(max(sload(p.ptr, kt + 1), e0), p.nnz);
+  }
+  if (wave8 >= 4) dkdv_run<true>(p, lds_base, kt, b, h, tid, lane, wave8, e0, e1, diag, part);
+  else            dkdv_run<false>(p, lds_base, kt, b, h, tid, lane, wave8, e0, e1, diag, part);
 }
 
 // dQ: one 64-key half tile for this wave's 32 query rows.
@@ -468,10 +507,23 @@ __global__ __launch_bounds__(256, 2) void dq_kernel(const BwdParams p) {
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int l32 = lane & 31, hi = lane >> 5;
   int pos, bh;
-  map_block(blockIdx.x, p.batch * p.n_heads, p.heads_per_xcd, p.n_qtiles, pos, bh);
-  const int qt = min(max(sload(p.order, pos), 0), p.n_qtiles - 1);
+  map_block(blockIdx.x, p.batch * p.n_heads, p.heads_per_xcd, p.n_qtiles * p.n_parts, pos, bh);
   const int b = bh / p.n_heads, h = bh % p.n_heads;
   const int64_t seq_q = (int64_t)p.n_qtiles * kTile;
+  int qt, e0, e1, diag = -1, part = 0;
+  if (p.dense) {
+    part = pos / p.n_qtiles;
+    const int line = pos - part * p.n_qtiles;
+    qt = p.dense_causal ? p.n_qtiles - 1 - line : line;    // longest rows first
+    if (p.dense_causal) diag = qt + p.diag_off;
+    const int kend = p.dense_causal ? min(max(diag + 1, 0), p.n_ktiles) : p.n_ktiles;
+    e0 = min(part * p.part_len, kend);
+    e1 = min(e0 + p.part_len, kend);
+  } else {
+    qt = min(max(sload(p.order, pos), 0), p.n_qtiles - 1);
+    e0 = min(max(sload(p.ptr, qt), 0), p.nnz);
+    e1 = min(max(sload(p.ptr, qt + 1), e0), p.nnz);
+  }
 
   const bf16* kbase = p.k + b * p.ks.b + h * p.ks.h;
   const bf16* vbase = p.v + b * p.vs.b + h * p.vs.h;
@@ -484,9 +536,9 @@ __global__ __launch_bounds__(256, 2) void dq_kernel(const BwdParams p) {
   const uint32_t v_extent = (uint32_t)((kTile - 1) * v_stride + kHeadDim) * 2;
   auto k_rsrc = [&](int kt) { return make_rsrc(kbase + (int64_t)kt * kTile * k_stride, k_extent); };
   auto v_rsrc = [&](int kt) { return make_rsrc(vbase + (int64_t)kt * kTile * v_stride, v_extent); };
-  auto ktile = [&](int e) { return min(max(sload(p.idx, e), 0), p.n_ktiles - 1); };
+  auto ktile = [&](int e) { return p.dense ? e : min(max(sload(p.idx, e), 0), p.n_ktiles - 1); };
+  auto is_causal = [&](int e) { return p.dense ? (int)(e == diag) : sload(p.flag, e); };
 
-  const int e0 = min(max(sload(p.ptr, qt), 0), p.nnz), e1 = min(max(sload(p.ptr, qt + 1), e0), p.nnz);
   int kt = e0 < e1 ? ktile(e0) : 0;
   if (e0 < e1) {
     dma_half_tile_buf<4>(sKA, k_rsrc(kt), koff, 0, wave);
@@ -513,7 +565,7 @@ __global__ __launch_bounds__(256, 2) void dq_kernel(const BwdParams p) {
   const TrLane tr(lane);
 
   for (int e = e0; e < e1; ++e) {
-    const int causal = sload(p.flag, e);
+    const int causal = is_causal(e);
     const int kt_next = e + 1 < e1 ? ktile(e + 1) : kt;
     wait_vmem_all();
     __syncthreads();            // stage A (keys 0..63) landed; everyone is done with stage B
@@ -532,7 +584,7 @@ __global__ __launch_bounds__(256, 2) void dq_kernel(const BwdParams p) {
       dq_half_tile(sKB, sVB, qf, dof, dq, tr, p.scale_log2, lse2, neg_delta, l32, hi, q_l, kHalf, causal);
     kt = kt_next;
   }
-  store_acc_t(p.out0 + b * p.o0s.b + (int64_t)qrow * p.o0s.s + h * p.o0s.h, dq, p.scale, hi);
+  store_result(p, p.out0, p.o0s, p.o0_part, part, b, qrow, h, seq_q, dq, p.scale, hi);
 }
 
 static int fill_common(BwdParams& p, const void* q, const void* k, const void* v, const void* dout,
@@ -544,8 +596,8 @@ static int fill_common(BwdParams& p, const void* q, const void* k, const void* v
   if (batch <= 0 || n_heads <= 0 || n_qtiles <= 0 || n_ktiles <= 0 || nnz < 0) return UA_ERR_SHAPE;
   if (nnz > 0 && (!idx || !flag)) return UA_ERR_NULL;          // only an empty list may leave them out
   if (flag && !aligned4(flag)) return UA_ERR_ALIGN;            // read one aligned 32-bit word at a time
-  if ((int64_t)batch * n_heads * n_qtiles > INT32_MAX || (int64_t)batch * n_heads * n_ktiles > INT32_MAX)
-    return UA_ERR_SHAPE;
+  if ((int64_t)batch * n_heads * n_qtiles * UA_MAX_PARTS > INT32_MAX ||
+      (int64_t)batch * n_heads * n_ktiles * UA_MAX_PARTS > INT32_MAX) return UA_ERR_SHAPE;
   if (head_dim != kHeadDim || !(softmax_scale > 0.f)) return UA_ERR_UNSUPPORTED;
   if (!aligned16(q) || !aligned16(k) || !aligned16(v) || !aligned16(dout)) return UA_ERR_ALIGN;
   if (!strides_ok(qs) || !strides_ok(ks) || !strides_ok(vs) || !strides_ok(ds)) return UA_ERR_ALIGN;
@@ -559,7 +611,18 @@ static int fill_common(BwdParams& p, const void* q, const void* k, const void* v
   p.scale = softmax_scale; p.scale_log2 = softmax_scale * kLog2e;
   const int nbh = batch * n_heads;
   p.heads_per_xcd = (nbh % 8 == 0) ? nbh / 8 : 0;
+  p.ptr = nullptr; p.idx = idx; p.flag = flag; p.order = nullptr;
+  p.dense = 0; p.dense_causal = 0; p.diag_off = 0; p.n_parts = 1; p.part_len = 0; p.out_f32 = 0; p.o0_part = 0; p.o1_part = 0;
   return check_device();
+}
+
+static int launch_dkdv(const BwdParams& p, hipStream_t st) {
+  hipLaunchKernelGGL(dkdv_kernel, dim3((unsigned)(p.batch * p.n_heads * p.n_ktiles * p.n_parts)), dim3(512), 0, st, p);
+  return hipGetLastError() == hipSuccess ? UA_OK : UA_ERR_LAUNCH;
+}
+static int launch_dq(const BwdParams& p, hipStream_t st) {
+  hipLaunchKernelGGL(dq_kernel, dim3((unsigned)(p.batch * p.n_heads * p.n_qtiles * p.n_parts)), dim3(256), 0, st, p);
+  return hipGetLastError() == hipSuccess ? UA_OK : UA_ERR_LAUNCH;
 }
 
 }  // namespace ua
@@ -582,8 +645,7 @@ extern "C" int ua_bsa_bwd_dkdv(const void* q, const void* k, const void* v, cons
   p.o0s = {dk_strides[0], dk_strides[1], dk_strides[2]};
   p.o1s = {dv_strides[0], dv_strides[1], dv_strides[2]};
   p.ptr = col_ptr; p.idx = row_idx; p.flag = cflag; p.order = k_order;
-  hipLaunchKernelGGL(dkdv_kernel, dim3((unsigned)(batch * n_heads * n_ktiles)), dim3(512), 0, (hipStream_t)stream, p);
-  return hipGetLastError() == hipSuccess ? UA_OK : UA_ERR_LAUNCH;
+  return launch_dkdv(p, (hipStream_t)stream);
 }
 
 extern "C" int ua_bsa_bwd_dq(const void* q, const void* k, const void* v, const void* dout,
@@ -604,6 +666,75 @@ extern "C" int ua_bsa_bwd_dq(const void* q, const void* k, const void* v, const 
   p.o0s = {dq_strides[0], dq_strides[1], dq_strides[2]};
   p.o1s = p.o0s;
   p.ptr = row_ptr; p.idx = col_idx; p.flag = flag; p.order = q_order;
-  hipLaunchKernelGGL(dq_kernel, dim3((unsigned)(batch * n_heads * n_qtiles)), dim3(256), 0, (hipStream_t)stream, p);
-  return hipGetLastError() == hipSuccess ? UA_OK : UA_ERR_LAUNCH;
+  return launch_dq(p, (hipStream_t)stream);
+}
+
+extern "C" int ua_dense_bwd(const void* dout, const void* q, const void* k, const void* v,
+                            const float* lse, const float* delta, void* dq, void* dk, void* dv,
+                            int batch, int n_heads, int seqlen_q, int seqlen_k, int head_dim,
+                            const int64_t* q_strides, const int64_t* k_strides, const int64_t* v_strides,
+                            const int64_t* do_strides, const int64_t* dq_strides, const int64_t* dk_strides,
+                            const int64_t* dv_strides, float softmax_scale, int causal,
+                            void* workspace, int64_t workspace_bytes, void* stream) {
+  using namespace ua;
+  if (seqlen_q <= 0 || seqlen_k <= 0 || seqlen_q % kTile || seqlen_k % kTile) return UA_ERR_SHAPE;
+  const int n_qtiles = seqlen_q / kTile, n_ktiles = seqlen_k / kTile;
+  BwdParams p;
+  if (int rc = fill_common(p, q, k, v, dout, lse, delta, nullptr, nullptr, batch, n_heads, n_qtiles, n_ktiles, 0,
+                           head_dim, q_strides, k_strides, v_strides, do_strides, softmax_scale)) return rc;
+  if (!dq || !dk || !dv || !dq_strides || !dk_strides || !dv_strides) return UA_ERR_NULL;
+  if (!aligned16(dq) || !aligned16(dk) || !aligned16(dv) || !strides_ok(dq_strides) || !strides_ok(dk_strides) ||
+      !strides_ok(dv_strides)) return UA_ERR_ALIGN;
+  hipStream_t st = (hipStream_t)stream;
+  p.dense = 1; p.dense_causal = causal != 0; p.diag_off = n_ktiles - n_qtiles;
+  const DenseSplit d = dense_split(batch, n_heads, n_qtiles, n_ktiles);
+  unsigned char* ws = static_cast<unsigned char*>(workspace);
+  const bool ws_ok = workspace && aligned16(workspace) && workspace_bytes >= d.bwd_total;
+  const void* parts[UA_MAX_PARTS];
+
+  // dK, dV: one workgroup per (key tile, head) walks the query tiles; few key tiles -> parts of the query range
+  {
+    BwdParams c = p;
+    c.out0 = (bf16*)dk; c.out1 = (bf16*)dv;
+    c.o0s = {dk_strides[0], dk_strides[1], dk_strides[2]};
+    c.o1s = {dv_strides[0], dv_strides[1], dv_strides[2]};
+    c.part_len = n_qtiles;
+    if (d.dkdv_parts > 1 && ws_ok) {
+      const int len = (n_qtiles + d.dkdv_parts - 1) / d.dkdv_parts;
+      const int n = (n_qtiles + len - 1) / len;
+      float* base = reinterpret_cast<float*>(ws);
+      ws += (int64_t)d.dkdv_parts * d.dkdv_bytes;
+      c.n_parts = n; c.part_len = len; c.out_f32 = 1;
+      c.o0_part = c.o1_part = d.dkdv_bytes / 4;
+      c.out0 = reinterpret_cast<bf16*>(base);
+      c.out1 = reinterpret_cast<bf16*>(base + d.dkdv_bytes / 8);
+      if (int rc = launch_dkdv(c, st)) return rc;
+      for (int i = 0; i < n; ++i) parts[i] = base + i * c.o0_part;
+      if (int rc = launch_grad_sum(parts, n, true, dk, dk_strides, batch, seqlen_k, n_heads, 1.f, st)) return rc;
+      for (int i = 0; i < n; ++i) parts[i] = base + d.dkdv_bytes / 8 + i * c.o1_part;
+      if (int rc = launch_grad_sum(parts, n, true, dv, dv_strides, batch, seqlen_k, n_heads, 1.f, st)) return rc;
+    } else if (int rc = launch_dkdv(c, st)) {
+      return rc;
+    }
+  }
+  // dQ: one workgroup per (query tile, head) walks the key tiles; few query tiles -> parts of the key range
+  {
+    BwdParams c = p;
+    c.out0 = (bf16*)dq; c.out1 = nullptr;
+    c.o0s = {dq_strides[0], dq_strides[1], dq_strides[2]};
+    c.o1s = c.o0s;
+    c.part_len = n_ktiles;
+    if (d.dq_parts > 1 && ws_ok) {
+      const int len = (n_ktiles + d.dq_parts - 1) / d.dq_parts;
+      const int n = (n_ktiles + len - 1) / len;
+      float* base = reinterpret_cast<float*>(ws);
+      c.n_parts = n; c.part_len = len; c.out_f32 = 1;
+      c.o0_part = d.dq_bytes / 4;
+      c.out0 = reinterpret_cast<bf16*>(base);
+      if (int rc = launch_dq(c, st)) return rc;
+      for (int i = 0; i < n; ++i) parts[i] = base + i * c.o0_part;
+      return launch_grad_sum(parts, n, true, dq, dq_strides, batch, seqlen_q, n_heads, 1.f, st);
+    }
+    return launch_dq(c, st);
+  }
 }

@@ -22,6 +22,12 @@ struct FwdParams {
   Strides3 qs, ks, vs, os;
   float scale_log2;      // softmax_scale * log2(e)
   int heads_per_xcd;     // batch*n_heads / 8 when divisible, else 0
+  // Dense rectangle (no list arrays): query tile qt walks key tiles [0, n_ktiles), or with
+  // dense_causal [0, qt + diag_off] with the last one causal.  The key range is cut into n_parts
+  // parts of part_len tiles; part i writes its partial (O, LSE) at o + i * o_part, lse + i * lse_part
+  // (elements).  Longest rows are launched first.
+  int dense, dense_causal, diag_off, n_parts, part_len;
+  int64_t o_part, lse_part;
 };
 
 constexpr int kHalf = 64;                          // keys per pipeline stage
@@ -142,14 +148,29 @@ __global__ __launch_bounds__(256, 2) void fwd_kernel(const FwdParams p) {
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int l32 = lane & 31, hi = lane >> 5;
   int pos, bh;
-  map_block(blockIdx.x, p.batch * p.n_heads, p.heads_per_xcd, p.n_qtiles, pos, bh);
-  const int qt = min(max(sload(p.q_order, pos), 0), p.n_qtiles - 1);
+  map_block(blockIdx.x, p.batch * p.n_heads, p.heads_per_xcd, p.n_qtiles * p.n_parts, pos, bh);
   const int b = bh / p.n_heads, h = bh % p.n_heads;
+  int qt, e0, e1, diag = -1, part = 0;
+  if (p.dense) {
+    part = pos / p.n_qtiles;
+    const int line = pos - part * p.n_qtiles;
+    qt = p.dense_causal ? p.n_qtiles - 1 - line : line;
+    if (p.dense_causal) diag = qt + p.diag_off;          // key tile on the diagonal (may lie outside the rectangle)
+    const int kend = p.dense_causal ? min(max(diag + 1, 0), p.n_ktiles) : p.n_ktiles;
+    e0 = min(part * p.part_len, kend);
+    e1 = min(e0 + p.part_len, kend);
+  } else {
+    qt = min(max(sload(p.q_order, pos), 0), p.n_qtiles - 1);
+    // list bounds are clamped to the arrays' extent: an inconsistent row_ptr cannot read beyond them
+    e0 = min(max(sload(p.row_ptr, qt), 0), p.nnz);
+    e1 = min(max(sload(p.row_ptr, qt + 1), e0), p.nnz);
+  }
+  // entry e of the walk: its key tile, and whether it is a causal tile
+  auto ktile = [&](int e) { return p.dense ? e : min(max(sload(p.col_idx, e), 0), p.n_ktiles - 1); };
+  auto is_causal = [&](int e) { return p.dense ? (int)(e == diag) : sload(p.flag, e); };
 
   const bf16* kbase = p.k + b * p.ks.b + h * p.ks.h;
   const bf16* vbase = p.v + b * p.vs.b + h * p.vs.h;
-  // list bounds are clamped to the arrays' extent: an inconsistent row_ptr cannot read beyond them
-  const int e0 = min(max(sload(p.row_ptr, qt), 0), p.nnz), e1 = min(max(sload(p.row_ptr, qt + 1), e0), p.nnz);
   const int k_stride = (int)p.ks.s, v_stride = (int)p.vs.s;
   int koff[4], voff[4];
   dma_voffsets<lds_off_k, 4>(koff, k_stride, wave, lane);
@@ -161,7 +182,7 @@ __global__ __launch_bounds__(256, 2) void fwd_kernel(const FwdParams p) {
   auto v_rsrc = [&](int kt) { return make_rsrc(vbase + (int64_t)kt * kTile * v_stride, v_extent); };
 
   // first half tile of the first entry goes in flight before anything else
-  int kt = e0 < e1 ? min(max(sload(p.col_idx, e0), 0), p.n_ktiles - 1) : 0;
+  int kt = e0 < e1 ? ktile(e0) : 0;
   if (e0 < e1) {
     dma_half_tile_buf<4>(sKA, k_rsrc(kt), koff, 0, wave);
     dma_half_tile_buf<4>(sVA, v_rsrc(kt), voff, 0, wave);
@@ -183,8 +204,8 @@ __global__ __launch_bounds__(256, 2) void fwd_kernel(const FwdParams p) {
   const TrLane tr(lane);
 
   for (int e = e0; e < e1; ++e) {
-    const int causal = sload(p.flag, e);
-    const int kt_next = e + 1 < e1 ? min(max(sload(p.col_idx, e + 1), 0), p.n_ktiles - 1) : kt;
+    const int causal = is_causal(e);
+    const int kt_next = e + 1 < e1 ? ktile(e + 1) : kt;
     // stage A (keys 0..63 of this tile) has landed; everyone is done with stage B
     wait_vmem_all();
     __syncthreads();
@@ -208,7 +229,7 @@ __global__ __launch_bounds__(256, 2) void fwd_kernel(const FwdParams p) {
   // ---- epilogue: normalise, write O (bf16) and LSE (natural log) -------------------------
   const float l_tot = xhalf_sum(st.l_run);
   const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
-  bf16* op = p.o + b * p.os.b + (int64_t)qrow * p.os.s + h * p.os.h;
+  bf16* op = p.o + part * p.o_part + b * p.os.b + (int64_t)qrow * p.os.s + h * p.os.h;
 #pragma unroll
   for (int mbd = 0; mbd < 4; ++mbd)
 #pragma unroll
@@ -220,8 +241,47 @@ __global__ __launch_bounds__(256, 2) void fwd_kernel(const FwdParams p) {
     }
   if (hi == 0) {
     const float lse = l_tot > 0.f ? (st.m_run + __builtin_amdgcn_logf(l_tot)) * kLn2 : -INFINITY;
-    p.lse[((int64_t)b * p.n_heads + h) * ((int64_t)p.n_qtiles * kTile) + qrow] = lse;
+    p.lse[part * p.lse_part + ((int64_t)b * p.n_heads + h) * ((int64_t)p.n_qtiles * kTile) + qrow] = lse;
   }
+}
+
+}  // namespace ua
+
+namespace ua {
+
+static int fwd_common(FwdParams& p, const void* q, const void* k, const void* v, void* o, float* lse,
+                      int batch, int n_heads, int n_qtiles, int n_ktiles, int head_dim,
+                      const int64_t* q_strides, const int64_t* k_strides, const int64_t* v_strides,
+                      const int64_t* o_strides, float softmax_scale) {
+  if (!q || !k || !v || !o || !lse || !q_strides || !k_strides || !v_strides || !o_strides) return UA_ERR_NULL;
+  if (batch <= 0 || n_heads <= 0 || n_qtiles <= 0 || n_ktiles <= 0) return UA_ERR_SHAPE;
+  if ((int64_t)batch * n_heads * n_qtiles * UA_MAX_PARTS > INT32_MAX) return UA_ERR_SHAPE;
+  if (head_dim != kHeadDim || !(softmax_scale > 0.f)) return UA_ERR_UNSUPPORTED;
+  if (!aligned16(q) || !aligned16(k) || !aligned16(v) || !aligned16(o)) return UA_ERR_ALIGN;
+  if (!strides_ok(q_strides) || !strides_ok(k_strides) || !strides_ok(v_strides) || !strides_ok(o_strides))
+    return UA_ERR_ALIGN;
+  if (k_strides[1] > (INT32_MAX >> 9) || v_strides[1] > (INT32_MAX >> 9)) return UA_ERR_SHAPE;
+  p.q = (const bf16*)q; p.k = (const bf16*)k; p.v = (const bf16*)v; p.o = (bf16*)o; p.lse = lse;
+  p.row_ptr = nullptr; p.col_idx = nullptr; p.flag = nullptr; p.q_order = nullptr;
+  p.batch = batch; p.n_heads = n_heads; p.n_qtiles = n_qtiles; p.n_ktiles = n_ktiles; p.nnz = 0;
+  p.qs = {q_strides[0], q_strides[1], q_strides[2]};
+  p.ks = {k_strides[0], k_strides[1], k_strides[2]};
+  p.vs = {v_strides[0], v_strides[1], v_strides[2]};
+  p.os = {o_strides[0], o_strides[1], o_strides[2]};
+  p.scale_log2 = softmax_scale * kLog2e;
+  const int nbh = batch * n_heads;
+  p.heads_per_xcd = (nbh % 8 == 0) ? nbh / 8 : 0;
+  p.dense = 0; p.dense_causal = 0; p.diag_off = 0; p.n_parts = 1; p.part_len = n_ktiles; p.o_part = 0; p.lse_part = 0;
+  return check_device();
+}
+
+static int fwd_launch(const FwdParams& p, hipStream_t st) {
+  hipLaunchKernelGGL(fwd_kernel, dim3((unsigned)(p.batch * p.n_heads * p.n_qtiles * p.n_parts)), dim3(256), 0, st, p);
+  return hipGetLastError() == hipSuccess ? UA_OK : UA_ERR_LAUNCH;
+}
+
+static bool contiguous_bshd(const int64_t* st, int seqlen, int n_heads) {
+  return st[2] == kHeadDim && st[1] == (int64_t)n_heads * kHeadDim && st[0] == (int64_t)seqlen * n_heads * kHeadDim;
 }
 
 }  // namespace ua
@@ -233,29 +293,53 @@ extern "C" int ua_bsa_fwd(const void* q, const void* k, const void* v, void* o, 
                           const int64_t* q_strides, const int64_t* k_strides, const int64_t* v_strides,
                           const int64_t* o_strides, float softmax_scale, void* stream) {
   using namespace ua;
-  if (!q || !k || !v || !o || !lse || !row_ptr || !q_order || !q_strides || !k_strides || !v_strides || !o_strides)
-    return UA_ERR_NULL;
-  if (batch <= 0 || n_heads <= 0 || n_qtiles <= 0 || n_ktiles <= 0 || nnz < 0) return UA_ERR_SHAPE;
+  if (!row_ptr || !q_order) return UA_ERR_NULL;
+  if (nnz < 0) return UA_ERR_SHAPE;
   if (nnz > 0 && (!col_idx || !flag)) return UA_ERR_NULL;      // only an empty list may leave them out
   if (flag && !aligned4(flag)) return UA_ERR_ALIGN;            // read one aligned 32-bit word at a time
-  if ((int64_t)batch * n_heads * n_qtiles > INT32_MAX) return UA_ERR_SHAPE;
-  if (head_dim != kHeadDim || !(softmax_scale > 0.f)) return UA_ERR_UNSUPPORTED;
-  if (!aligned16(q) || !aligned16(k) || !aligned16(v) || !aligned16(o)) return UA_ERR_ALIGN;
-  if (!strides_ok(q_strides) || !strides_ok(k_strides) || !strides_ok(v_strides) || !strides_ok(o_strides))
-    return UA_ERR_ALIGN;
-  if (k_strides[1] > (INT32_MAX >> 9) || v_strides[1] > (INT32_MAX >> 9)) return UA_ERR_SHAPE;
-  if (int rc = check_device()) return rc;
   FwdParams p;
-  p.q = (const bf16*)q; p.k = (const bf16*)k; p.v = (const bf16*)v; p.o = (bf16*)o; p.lse = lse;
-  p.row_ptr = row_ptr; p.col_idx = col_idx; p.flag = flag; p.q_order = q_order;
-  p.batch = batch; p.n_heads = n_heads; p.n_qtiles = n_qtiles; p.n_ktiles = n_ktiles; p.nnz = nnz;
-  p.qs = {q_strides[0], q_strides[1], q_strides[2]};
-  p.ks = {k_strides[0], k_strides[1], k_strides[2]};
-  p.vs = {v_strides[0], v_strides[1], v_strides[2]};
-  p.os = {o_strides[0], o_strides[1], o_strides[2]};
-  p.scale_log2 = softmax_scale * kLog2e;
-  const int nbh = batch * n_heads;
-  p.heads_per_xcd = (nbh % 8 == 0) ? nbh / 8 : 0;
-  hipLaunchKernelGGL(fwd_kernel, dim3((unsigned)(nbh * n_qtiles)), dim3(256), 0, (hipStream_t)stream, p);
-  return hipGetLastError() == hipSuccess ? UA_OK : UA_ERR_LAUNCH;
+  if (int rc = fwd_common(p, q, k, v, o, lse, batch, n_heads, n_qtiles, n_ktiles, head_dim, q_strides, k_strides,
+                          v_strides, o_strides, softmax_scale)) return rc;
+  p.row_ptr = row_ptr; p.col_idx = col_idx; p.flag = flag; p.q_order = q_order; p.nnz = nnz;
+  return fwd_launch(p, (hipStream_t)stream);
+}
+
+extern "C" int64_t ua_dense_workspace_bytes(int batch, int n_heads, int seqlen_q, int seqlen_k, int backward) {
+  using namespace ua;
+  if (batch <= 0 || n_heads <= 0 || seqlen_q <= 0 || seqlen_k <= 0 || seqlen_q % kTile || seqlen_k % kTile) return 0;
+  const DenseSplit d = dense_split(batch, n_heads, seqlen_q / kTile, seqlen_k / kTile);
+  return backward ? d.bwd_total : d.fwd_total;
+}
+
+extern "C" int ua_dense_fwd(const void* q, const void* k, const void* v, void* o, float* lse,
+                            int batch, int n_heads, int seqlen_q, int seqlen_k, int head_dim,
+                            const int64_t* q_strides, const int64_t* k_strides, const int64_t* v_strides,
+                            const int64_t* o_strides, float softmax_scale, int causal,
+                            void* workspace, int64_t workspace_bytes, void* stream) {
+  using namespace ua;
+  if (seqlen_q <= 0 || seqlen_k <= 0 || seqlen_q % kTile || seqlen_k % kTile) return UA_ERR_SHAPE;
+  const int n_qtiles = seqlen_q / kTile, n_ktiles = seqlen_k / kTile;
+  FwdParams p;
+  if (int rc = fwd_common(p, q, k, v, o, lse, batch, n_heads, n_qtiles, n_ktiles, head_dim, q_strides, k_strides,
+                          v_strides, o_strides, softmax_scale)) return rc;
+  p.dense = 1; p.dense_causal = causal != 0; p.diag_off = n_ktiles - n_qtiles;
+  hipStream_t st = (hipStream_t)stream;
+  const DenseSplit d = dense_split(batch, n_heads, n_qtiles, n_ktiles);
+  // the split path needs the caller's workspace and a contiguous output for the merge
+  const bool split = d.fwd_parts > 1 && workspace && aligned16(workspace) && workspace_bytes >= d.fwd_total &&
+                     contiguous_bshd(o_strides, seqlen_q, n_heads);
+  if (!split) return fwd_launch(p, st);
+  const int len = (n_ktiles + d.fwd_parts - 1) / d.fwd_parts;
+  const int parts = (n_ktiles + len - 1) / len;
+  unsigned char* ws = static_cast<unsigned char*>(workspace);
+  p.o = reinterpret_cast<bf16*>(ws);
+  p.lse = reinterpret_cast<float*>(ws + (int64_t)parts * d.fwd_o_bytes);
+  p.o_part = d.fwd_o_bytes / 2; p.lse_part = d.fwd_lse_bytes / 4;
+  p.os = {(int64_t)seqlen_q * n_heads * kHeadDim, (int64_t)n_heads * kHeadDim, kHeadDim};
+  p.n_parts = parts; p.part_len = len;
+  if (int rc = fwd_launch(p, st)) return rc;
+  const void* op[UA_MAX_PARTS];
+  const float* lp[UA_MAX_PARTS];
+  for (int i = 0; i < parts; ++i) { op[i] = p.o + i * p.o_part; lp[i] = p.lse + i * p.lse_part; }
+  return ua_merge(op, lp, parts, o, lse, batch, seqlen_q, n_heads, head_dim, stream);
 }

@@ -170,4 +170,43 @@ inline bool strides_ok(const int64_t* s) { return s && s[0] % 8 == 0 && s[1] % 8
 
 int check_device();   // UA_OK when the current device is gfx950
 
+// ---- dense rectangles: how many parts a walk is cut into -------------------------------------
+// A dense rectangle launches one workgroup per (tile line, head); with few lines and heads the
+// device (256 CUs, two resident workgroups each for the row walks) stays empty while every
+// workgroup walks a long list.  The walk is then cut into parts that run as workgroups of their
+// own and leave partial results, combined by a second, HBM-bound kernel.  No split when the launch
+// fills the device anyway or the list is short; else enough parts for ~2 workgroups per CU, at
+// least two tiles each, at most UA_MAX_PARTS.
+constexpr int kDenseFullLaunch = 384, kDenseTargetGroups = 512;
+inline int dense_parts(int64_t n_workgroups, int list_len) {
+  if (n_workgroups >= kDenseFullLaunch || list_len < 4) return 1;
+  int64_t want = (kDenseTargetGroups + n_workgroups - 1) / n_workgroups;
+  if (want > UA_MAX_PARTS) want = UA_MAX_PARTS;
+  if (want > list_len / 2) want = list_len / 2;
+  return want >= 2 ? (int)want : 1;
+}
+inline int64_t align256(int64_t x) { return (x + 255) / 256 * 256; }
+struct DenseSplit {     // parts and workspace layout of one dense call (bytes, 256-byte aligned blocks)
+  int fwd_parts, dq_parts, dkdv_parts;
+  int64_t fwd_o_bytes, fwd_lse_bytes;          // per part
+  int64_t dq_bytes, dkdv_bytes;                // per part (dkdv: dK then dV)
+  int64_t fwd_total, bwd_total;
+};
+inline DenseSplit dense_split(int batch, int n_heads, int n_qtiles, int n_ktiles) {
+  DenseSplit d;
+  const int64_t nbh = (int64_t)batch * n_heads;
+  d.fwd_parts = d.dq_parts = dense_parts(nbh * n_qtiles, n_ktiles);
+  d.dkdv_parts = dense_parts(nbh * n_ktiles * 2, n_qtiles);      // one dK/dV workgroup fills a CU
+  const int64_t q_elems = nbh * n_qtiles * kTile * kHeadDim, k_elems = nbh * n_ktiles * kTile * kHeadDim;
+  d.fwd_o_bytes = align256(q_elems * 2);
+  d.fwd_lse_bytes = align256(nbh * n_qtiles * kTile * 4);
+  d.dq_bytes = align256(q_elems * 4);
+  d.dkdv_bytes = 2 * align256(k_elems * 4);
+  d.fwd_total = d.fwd_parts > 1 ? d.fwd_parts * (d.fwd_o_bytes + d.fwd_lse_bytes) : 0;
+  d.bwd_total = (d.dq_parts > 1 ? d.dq_parts * d.dq_bytes : 0) + (d.dkdv_parts > 1 ? d.dkdv_parts * d.dkdv_bytes : 0);
+  return d;
+}
+int launch_grad_sum(const void* const* parts, int n_parts, bool parts_fp32, void* out, const int64_t* out_strides,
+                    int batch, int seqlen, int n_heads, float scale, hipStream_t st);
+
 }  // namespace ua

@@ -40,10 +40,12 @@ def format_entry(S: int, Nh: int, causal: bool, ratio: Tuple[int, int], fwd_us: 
             [round(fwd_us, 3), round(bwd_us, 3), round(flops / fwd_us / 1e6, 3), round(2.5 * flops / bwd_us / 1e6, 3)]]
 
 
-def time_tile(S: int, Nh: int, causal: bool, ratio: Tuple[int, int] = (1, 1), budget_s: float = 0.25, D: int = HEAD_DIM):
+def time_tile(S: int, Nh: int, causal: bool, ratio: Tuple[int, int] = (1, 1), budget_s: float = 0.25, D: int = HEAD_DIM,
+              use_graph: bool = True):
     """(fwd us, bwd us) of one dense ``Sq x Skv`` tile, Sq = S*r, Skv = S*c, through the drop-in
-    ``_flash_attn_forward`` / ``_flash_attn_backward``; the iteration count follows a first
-    timed launch so that every shape costs about ``budget_s`` per direction."""
+    ``_flash_attn_forward`` / ``_flash_attn_backward`` (``ua_dense_fwd`` / ``ua_dense_bwd``, which cut
+    rectangles with few tile lines into parts); the iteration count follows a first timed launch so
+    that every shape costs about ``budget_s`` per direction."""
     import torch
     from .flash_attn_interface import _flash_attn_backward, _flash_attn_forward
     from .ops import softmax_delta
@@ -66,11 +68,28 @@ def time_tile(S: int, Nh: int, causal: bool, ratio: Tuple[int, int] = (1, 1), bu
     torch.cuda.synchronize()
 
     def timed(fn, iters):
+        """us per call.  The calls are recorded into one HIP graph and the graph's replay is timed,
+        so that what is measured is the device's time per call (kernels and the gaps between
+        dependent launches) and not the host's cost of issuing a call from Python, which for tiles
+        of a few microseconds would be all that is seen."""
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        e0.record()
-        for _ in range(iters):
-            fn()
-        e1.record()
+        if use_graph:
+            side = torch.cuda.Stream()
+            side.wait_stream(torch.cuda.current_stream())
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph, stream=side):
+                for _ in range(iters):
+                    fn()
+            graph.replay()
+            torch.cuda.synchronize()
+            e0.record()
+            graph.replay()
+            e1.record()
+        else:
+            e0.record()
+            for _ in range(iters):
+                fn()
+            e1.record()
         torch.cuda.synchronize()
         return e0.elapsed_time(e1) / iters * 1e3                     # us
     out = []
