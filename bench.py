@@ -41,13 +41,24 @@ def load_traffic():
             TRAFFIC_BYTES[(w, m.group(1))] = (float(m.group(2)) * 1e9, os.path.relpath(path, ROOT))
 
 
-def roof_entry(workload, kernel, bound, achieved, peak, unit, kernel_ms, algorithmic):
+MEASURED_MFMA_CEILING = [None]     # TFLOP/s, set from this run's own register-only MFMA probe
+
+
+def roof_entry(workload, kernel, bound, achieved, peak, unit, kernel_ms, algorithmic, kernel_ms_min=None):
+    """`achieved`, `kernel_ms`: median over the repeats of the timed block; `*_min`: the best repeat."""
     tr = TRAFFIC_BYTES.get((workload, kernel))
     e = {"workload": workload, "kernel": kernel, "bound": bound, "achieved": achieved, "peak": peak, "unit": unit,
          "frac": achieved / peak, "kernel_ms": kernel_ms,
          "traffic": tr[0] if tr else None,
          "traffic_source": (tr[1] + " (rocprofv3 --pmc, a constant from that file, not measured in this run)") if tr else None}
     e["algorithmic_flops" if bound == "mfma" else "algorithmic_bytes"] = algorithmic
+    if kernel_ms_min:
+        e["kernel_ms_min"] = kernel_ms_min
+        e["achieved_best"] = achieved * kernel_ms / kernel_ms_min
+    if bound == "mfma" and MEASURED_MFMA_CEILING[0]:
+        # against what the matrix pipes of THIS device deliver to a register-only loop on random bf16 data
+        e["measured_mfma_ceiling"] = MEASURED_MFMA_CEILING[0]
+        e["frac_of_measured_mfma_ceiling"] = achieved / MEASURED_MFMA_CEILING[0]
     return e
 
 
@@ -55,16 +66,33 @@ def attention_roofs(workload, res, peak):
     """Roofline entries of the attention kernels of one workload result (algorithmic flops by the
     reference's convention: forward F, dK/dV 4 of the backward's 5 GEMMs = 2.0 F, dQ 1 of 5 = 0.5 F)."""
     F = res["fwd_flops"]
+    mn = res.get("min", {})
     launches = 4 if workload == "c5" else 1          # c5 runs the forward as 4 kernel tiles
-    out = [roof_entry(workload, "fwd_kernel", "mfma", res["fwd_tflops"], peak, "TFLOP/s", res["fwd_ms"] / launches, F / launches)]
+    per = lambda key: mn[key] / launches if key in mn else None
+    out = [roof_entry(workload, "fwd_kernel", "mfma", res["fwd_tflops"], peak, "TFLOP/s", res["fwd_ms"] / launches, F / launches,
+                      per("fwd_ms"))]
     if "dkdv_ms" in res:
-        out.append(roof_entry(workload, "dkdv_kernel", "mfma", 2.0 * F / res["dkdv_ms"] / 1e9, peak, "TFLOP/s", res["dkdv_ms"], 2.0 * F))
-        out.append(roof_entry(workload, "dq_kernel", "mfma", 0.5 * F / res["dq_ms"] / 1e9, peak, "TFLOP/s", res["dq_ms"], 0.5 * F))
+        out.append(roof_entry(workload, "dkdv_kernel", "mfma", 2.0 * F / res["dkdv_ms"] / 1e9, peak, "TFLOP/s", res["dkdv_ms"], 2.0 * F,
+                              mn.get("dkdv_ms")))
+        out.append(roof_entry(workload, "dq_kernel", "mfma", 0.5 * F / res["dq_ms"] / 1e9, peak, "TFLOP/s", res["dq_ms"], 0.5 * F,
+                              mn.get("dq_ms")))
         nbytes = res["delta_gbps"] * res["delta_ms"] * 1e6
-        out.append(roof_entry(workload, "delta_kernel", "hbm", res["delta_gbps"], HBM_PEAK_GBPS, "GB/s", res["delta_ms"], nbytes))
+        out.append(roof_entry(workload, "delta_kernel", "hbm", res["delta_gbps"], HBM_PEAK_GBPS, "GB/s", res["delta_ms"], nbytes,
+                              mn.get("delta_ms")))
     if "merge_ms" in res:
-        out.append(roof_entry(workload, "merge_kernel<4>", "hbm", res["merge_gbps"], HBM_PEAK_GBPS, "GB/s", res["merge_ms"], res["merge_bytes"]))
+        out.append(roof_entry(workload, "merge_kernel<4>", "hbm", res["merge_gbps"], HBM_PEAK_GBPS, "GB/s", res["merge_ms"],
+                              res["merge_bytes"], mn.get("merge_ms")))
     return out
+
+
+REPEATS = 3          # the reference's protocol: warm-up, then 3 repeats of the timed block (search_algo/benchmark.py:197-216)
+
+
+def median_min(repeats):
+    """repeats: list of {name: ms}.  -> ({name: median}, {name: min})"""
+    keys = repeats[0].keys()
+    med = {k: sorted(r[k] for r in repeats)[len(repeats) // 2] for k in keys}
+    return med, {k: min(r[k] for r in repeats) for k in keys}
 
 
 def log(*a):
@@ -86,6 +114,7 @@ def probe_lib():
         vp, ci = ctypes.c_void_p, ctypes.c_int
         lib.bench_probe_mfma.restype, lib.bench_probe_mfma.argtypes = ci, [vp, vp, ci, ci, vp]
         lib.bench_probe_mfma_rotating.restype, lib.bench_probe_mfma_rotating.argtypes = ci, [vp, vp, ci, ci, vp]
+        lib.bench_probe_mfma16_rotating.restype, lib.bench_probe_mfma16_rotating.argtypes = ci, [vp, vp, ci, ci, vp]
         lib.bench_atomic_rate.restype, lib.bench_atomic_rate.argtypes = ci, [vp, ctypes.c_int64, ci, ci, ci, vp]
         lib.bench_stream_mix.restype = ci
         lib.bench_stream_mix.argtypes = [ctypes.POINTER(vp), ci, vp, ctypes.c_int64, ci, ci, vp]
@@ -164,21 +193,27 @@ def run_attention(name, steps, warmup, backward):
     for _ in range(warmup):
         step()
     torch.cuda.synchronize()
-    timer = Timer(torch, names)
-    t0 = time.perf_counter()
-    for _ in range(steps):
-        step(timer)
-    torch.cuda.synchronize()
-    wall_ms = (time.perf_counter() - t0) * 1e3 / steps
-    timer.collect()
+    reps = []
+    for _ in range(REPEATS):                  # each repeat times exactly `steps` steps
+        timer = Timer(torch, names)
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            step(timer)
+        torch.cuda.synchronize()
+        rep = {"ms_per_step": (time.perf_counter() - t0) * 1e3 / steps}
+        timer.collect()
+        rep.update({n + "_ms": timer.acc[n] / steps for n in names})
+        reps.append(rep)
+    ms, mn = median_min(reps)
+    wall_ms = ms["ms_per_step"]
     F = fwd_flops(mask)
-    ms = {n: timer.acc[n] / steps for n in names}
     res = {"workload": name, "tiles_per_head": tl.nnz, "tilelist_sha256": tl.sha256(), "tilelist_build_ms": t_build * 1e3,
-           "ms_per_step": wall_ms, "fwd_ms": ms["fwd"], "fwd_tflops": F / ms["fwd"] / 1e9, "fwd_flops": F}
+           "ms_per_step": wall_ms, "fwd_ms": ms["fwd_ms"], "fwd_tflops": F / ms["fwd_ms"] / 1e9, "fwd_flops": F,
+           "repeats": reps, "min": mn, "fwd_tflops_best": F / mn["fwd_ms"] / 1e9}
     if backward:
-        res.update(bwd_ms=ms["bwd"], delta_ms=ms["delta"], bwd_tflops=2.5 * F / (ms["bwd"] + ms["delta"]) / 1e9,
-                   fwd_bwd_tflops=3.5 * F / wall_ms / 1e9,
-                   delta_gbps=(2 * q.numel() * 2 + lse.numel() * 4) / ms["delta"] / 1e6)
+        res.update(bwd_ms=ms["bwd_ms"], delta_ms=ms["delta_ms"], bwd_tflops=2.5 * F / (ms["bwd_ms"] + ms["delta_ms"]) / 1e9,
+                   fwd_bwd_tflops=3.5 * F / wall_ms / 1e9, fwd_bwd_tflops_best=3.5 * F / mn["ms_per_step"] / 1e9,
+                   delta_gbps=(2 * q.numel() * 2 + lse.numel() * 4) / ms["delta_ms"] / 1e6)
     return res
 
 
@@ -216,12 +251,15 @@ def time_bwd_kernels(name, steps):
                                      tl.n_ktiles, tl.nnz, 128, s3(q), s3(k), s3(v), s3(do), s3(dq), SCALE, st), "dq")
     dkdv(); dqk()
     torch.cuda.synchronize()
-    t = Timer(torch, ["dkdv", "dq"])
-    for _ in range(steps):
-        t.mark(); dkdv(); t.mark(); dqk(); t.mark()
-    torch.cuda.synchronize()
-    t.collect()
-    return {n: t.acc[n] / steps for n in t.names}
+    reps = []
+    for _ in range(REPEATS):
+        t = Timer(torch, ["dkdv", "dq"])
+        for _ in range(steps):
+            t.mark(); dkdv(); t.mark(); dqk(); t.mark()
+        torch.cuda.synchronize()
+        t.collect()
+        reps.append({n + "_ms": t.acc[n] / steps for n in t.names})
+    return median_min(reps)
 
 
 def run_c5(steps, warmup):
@@ -257,17 +295,23 @@ def run_c5(steps, warmup):
     for _ in range(warmup):
         step()
     torch.cuda.synchronize()
-    timer = Timer(torch, ["fwd_tiles", "merge"])
-    t0 = time.perf_counter()
-    for _ in range(steps):
-        step(timer)
-    torch.cuda.synchronize()
-    wall_ms = (time.perf_counter() - t0) * 1e3 / steps
-    timer.collect()
+    reps = []
+    for _ in range(REPEATS):
+        timer = Timer(torch, ["fwd_tiles", "merge"])
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            step(timer)
+        torch.cuda.synchronize()
+        rep = {"ms_per_step": (time.perf_counter() - t0) * 1e3 / steps}
+        timer.collect()
+        rep.update(fwd_ms=timer.acc["fwd_tiles"] / steps, merge_ms=timer.acc["merge"] / steps)
+        reps.append(rep)
+    med, mn = median_min(reps)
+    wall_ms = med["ms_per_step"]
     F = fwd_flops(mask)
     rows = nqb * BLOCK * HEADS
     merge_bytes = (len(tls) + 1) * rows * (128 * 2 + 4)
-    m_ms, f_ms = timer.acc["merge"] / steps, timer.acc["fwd_tiles"] / steps
+    m_ms, f_ms = med["merge_ms"], med["fwd_ms"]
     # the device's rate for the merge's memory pattern without its arithmetic: 4 streams read, 1 written,
     # 16-byte accesses, one load step per workgroup, on the same buffers
     import ctypes
@@ -287,7 +331,8 @@ def run_c5(steps, warmup):
     return {"workload": "c5", "stream_mix_4r1w_gbps": mix_gbps, "merge_frac_of_stream_mix": merge_bytes / m_ms / 1e6 / mix_gbps, "ms_per_step": wall_ms, "fwd_ms": f_ms, "fwd_tflops": F / f_ms / 1e9, "fwd_flops": F,
             "merge_ms": m_ms, "merge_bytes": merge_bytes, "merge_gbps": merge_bytes / m_ms / 1e6,
             "merge_frac_of_hbm": merge_bytes / m_ms / 1e6 / HBM_PEAK_GBPS,
-            "fwd_plus_merge_tflops": F / wall_ms / 1e9}
+            "merge_gbps_best": merge_bytes / mn["merge_ms"] / 1e6,
+            "fwd_plus_merge_tflops": F / wall_ms / 1e9, "repeats": reps, "min": mn}
 
 
 def run_mask_builder(name, steps):
@@ -311,7 +356,7 @@ def run_mask_builder(name, steps):
     ms = e0.elapsed_time(e1) / steps
     nbytes = mask.size + 2 * host.nnz * 5 + 4 * (2 * (host.n_qtiles + host.n_ktiles) + 2)
     return {"workload": name, "ms": ms, "bytes": nbytes, "gbps": nbytes / ms / 1e6, "nnz_tiles": host.nnz,
-            "matches_host_builder": same, "note": "latency-bound: 8 dependent launches over a few MB"}
+            "matches_host_builder": same, "note": "latency-bound: 11 small dependent launches over a few MB"}
 
 
 def run_cols_gather(steps):
@@ -430,21 +475,29 @@ def run_power(name):
 
 
 def probe_mfma(peak):
-    """Sustained register-only MFMA rate with constant and with random operand bits."""
+    """Sustained register-only MFMA rates: constant and random operand bits; both dense bf16
+    instructions (32x32x16 and 16x16x32) with operands that change on every instruction, at 1 and at
+    2 waves per SIMD.  `measured_ceiling_tflops` = the best of the random-data figures: what the
+    matrix pipes of this device deliver to any bf16 kernel fed with ordinary data."""
     import torch
     lib = probe_lib()
     dev = "cuda:0"
-    n_blocks, iters = 512, 40000
-    out = torch.empty(n_blocks * 256, dtype=torch.float32, device=dev)
+    out = torch.empty(512 * 256, dtype=torch.float32, device=dev)
     g = torch.Generator(device=dev).manual_seed(0)
     ops_ = {"constant": torch.ones(512 * 8, dtype=torch.bfloat16, device=dev),
             "random": torch.randn(512 * 8, dtype=torch.float32, device=dev, generator=g).to(torch.bfloat16)}
     res = {}
     st = torch.cuda.current_stream().cuda_stream
     rot = torch.randn(16 * 256 * 8, dtype=torch.float32, device=dev, generator=g).to(torch.bfloat16)
-    runs = [(name + "_operands_tflops", lib.bench_probe_mfma, t) for name, t in ops_.items()]
-    runs.append(("rotating_random_operands_tflops", lib.bench_probe_mfma_rotating, rot))
-    for key, fn, t in runs:
+    # (key, entry point, operands, workgroups of 4 waves, iterations, flop per thread-iteration / 64 lanes)
+    f32 = 4 * 32768.0          # 4 MFMAs of 32x32x16 per wave and iteration
+    f16 = 8 * 16384.0          # 8 MFMAs of 16x16x32
+    runs = [(name + "_operands_tflops", lib.bench_probe_mfma, t, 512, 40000, f32) for name, t in ops_.items()]
+    runs += [("rotating_random_operands_tflops", lib.bench_probe_mfma_rotating, rot, 512, 40000, f32),
+             ("rotating_random_1_wave_per_simd_tflops", lib.bench_probe_mfma_rotating, rot, 256, 80000, f32),
+             ("rotating_random_16x16x32_tflops", lib.bench_probe_mfma16_rotating, rot, 512, 40000, f16),
+             ("rotating_random_16x16x32_1_wave_per_simd_tflops", lib.bench_probe_mfma16_rotating, rot, 256, 80000, f16)]
+    for key, fn, t, n_blocks, iters, flop in runs:
         assert fn(t.data_ptr(), out.data_ptr(), n_blocks, 2000, st) == 0
         torch.cuda.synchronize()
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
@@ -452,14 +505,42 @@ def probe_mfma(peak):
         assert fn(t.data_ptr(), out.data_ptr(), n_blocks, iters, st) == 0
         e1.record()
         torch.cuda.synchronize()
-        ms = e0.elapsed_time(e1)
-        res[key] = n_blocks * 4 * 4 * iters * 32768.0 / ms / 1e9
+        res[key] = n_blocks * 4 * iters * flop / e0.elapsed_time(e1) / 1e9
     res["frac_of_peak_random"] = res["random_operands_tflops"] / peak
-    res["note"] = ("register-only v_mfma_f32_32x32x16_bf16 loops, 2 waves per SIMD: one A/B operand pair reused for ever "
-                   "(constant bits, random N(0,1) bits) and 8x8 random fragments cycled so that the operands change on "
-                   "every instruction; the clock follows power, power follows operand bit activity, so the random "
-                   "figure is the practical ceiling of any bf16 MFMA kernel on this device")
+    res["measured_ceiling_tflops"] = max(v for k, v in res.items() if "random" in k and k.endswith("_tflops"))
+    res["measured_ceiling_frac_of_peak"] = res["measured_ceiling_tflops"] / peak
+    res["note"] = ("register-only MFMA loops, 512 (2 waves per SIMD) or 256 (1 wave per SIMD) workgroups of 4 waves: one A/B "
+                   "operand pair reused for ever (constant bits, random N(0,1) bits), and 8x8 random fragments cycled so that "
+                   "the operands change on every instruction, for v_mfma_f32_32x32x16_bf16 and v_mfma_f32_16x16x32_bf16; the "
+                   "clock follows power, power follows operand bit activity, so the best random figure is the practical "
+                   "ceiling of any bf16 MFMA kernel on this device")
     return res
+
+
+def run_grad_accumulate(steps):
+    """One step of the gradient packs' fp32 accumulation at the 128k shape ([dK | dV] of one device:
+    2 x 131072 x 32 x 128 elements): reads fp32 + bf16, writes fp32 + bf16 = 12 bytes per element."""
+    import torch
+    from ultraattn_amd import ops
+    n = 2 * 131072 * HEADS * 128
+    acc = torch.zeros(n, dtype=torch.float32, device="cuda:0")
+    part = torch.empty(n, dtype=torch.bfloat16, device="cuda:0").normal_()
+    out = torch.empty_like(part)
+    ops.grad_accumulate(part, out, acc=acc)
+    torch.cuda.synchronize()
+    reps = []
+    for _ in range(REPEATS):
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(steps):
+            ops.grad_accumulate(part, out, acc=acc)
+        e1.record()
+        torch.cuda.synchronize()
+        reps.append({"ms": e0.elapsed_time(e1) / steps})
+    med, mn = median_min(reps)
+    return {"ms": med["ms"], "ms_min": mn["ms"], "bytes": 12 * n, "gbps": 12 * n / med["ms"] / 1e6,
+            "frac_of_hbm": 12 * n / med["ms"] / 1e6 / HBM_PEAK_GBPS,
+            "shape": "acc fp32 += partial bf16, out bf16 = round(acc); 2 x 131072 x 32 x 128 elements"}
 
 
 def device_ceilings(peak):
@@ -548,6 +629,16 @@ def device_ceilings(peak):
     return out
 
 
+def cpu_model():
+    try:
+        for line in open("/proc/cpuinfo"):
+            if line.startswith("model name"):
+                return line.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    return "unknown"
+
+
 def cpu_baseline():
     """The reference's block-loop path restated on the CPU (oracle.block_loop_fwd), timed on
     config 1 exactly: B=1, S=8192, Nh=8, d=128, fp32, 16x16 causal block grid, forward only."""
@@ -570,7 +661,7 @@ def cpu_baseline():
     return {"value": F / best / 1e12, "unit": "TFLOP/s", "cores": torch.get_num_threads(), "kind": "port",
             "sample": "config 1 whole: B=1 S=8192 Nh=8 d=128 fp32 causal 16x16 blocks of 512, forward, "
                       f"{len(timed)} runs, min {best:.3f} s, median {sorted(timed)[len(timed) // 2]:.3f} s",
-            "affinity_cores": len(os.sched_getaffinity(0)), "flops": F,
+            "affinity_cores": len(os.sched_getaffinity(0)), "cpu_model": cpu_model(), "flops": F,
             "parity": config1_parity(ao, mask, q, k, v)}
 
 
@@ -631,6 +722,9 @@ def main():
         dst.copy_(src)
         torch.cuda.synchronize()
         del src, dst
+    mfma_probe = probe_mfma(peak)
+    MEASURED_MFMA_CEILING[0] = mfma_probe["measured_ceiling_tflops"]
+    log(json.dumps(mfma_probe))
     if a.workload == "c5":
         main_res = run_c5(a.steps, a.warmup)
     else:
@@ -639,15 +733,17 @@ def main():
     load_traffic()
     backward = "fwd_bwd_tflops" in main_res
     if backward:
-        kt = time_bwd_kernels(a.workload, max(3, a.steps // 2))
+        kt, kt_min = time_bwd_kernels(a.workload, max(3, a.steps // 2))
         F = main_res["fwd_flops"]
-        main_res.update(dkdv_ms=kt["dkdv"], dq_ms=kt["dq"], dkdv_tflops=2.0 * F / kt["dkdv"] / 1e9,
-                        dq_tflops=0.5 * F / kt["dq"] / 1e9)
+        main_res.update(dkdv_ms=kt["dkdv_ms"], dq_ms=kt["dq_ms"], dkdv_tflops=2.0 * F / kt["dkdv_ms"] / 1e9,
+                        dq_tflops=0.5 * F / kt["dq_ms"] / 1e9)
+        main_res["min"].update(kt_min)
         value = main_res["fwd_bwd_tflops"]
         metric = "effective TFLOP/s on active blocks, forward+backward"
     else:
         value = main_res.get("fwd_plus_merge_tflops", main_res["fwd_tflops"])
         metric = "effective TFLOP/s on active blocks, forward"
+    value_best = value * main_res["ms_per_step"] / main_res["min"]["ms_per_step"]
     roofs = attention_roofs(a.workload, main_res, peak)
     # the dominant kernel of the step: dK/dV for the forward+backward workloads, the forward otherwise
     roof = dict(next(r for r in roofs if r["kernel"] == ("dkdv_kernel" if backward else "fwd_kernel")))
@@ -662,10 +758,11 @@ def main():
                 run_attention(w, max(3, a.steps // 2), 2, backward=w in ("c3", "c4"))
             if "fwd_bwd_tflops" in r:
                 torch.cuda.empty_cache()
-                kt = time_bwd_kernels(w, 3)
-                r.update(dkdv_ms=kt["dkdv"], dq_ms=kt["dq"])
+                kt, kt_min = time_bwd_kernels(w, 3)
+                r.update(dkdv_ms=kt["dkdv_ms"], dq_ms=kt["dq_ms"])
+                r["min"].update(kt_min)
             roofs += attention_roofs(w, r, peak)
-            for key in ("tilelist_sha256", "fwd_flops"):
+            for key in ("tilelist_sha256", "fwd_flops", "repeats"):
                 r.pop(key, None)
             r["fwd_frac_of_peak"] = r["fwd_tflops"] / peak
             if "fwd_bwd_tflops" in r:
@@ -673,7 +770,8 @@ def main():
             extra[w] = r
             log(json.dumps(r))
     out = {"metric": metric, "value": value, "unit": "TFLOP/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
-           "ms_per_step": main_res["ms_per_step"], "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+           "repeats": REPEATS, "value_is": "median over the repeats of the timed block of `steps` steps", "value_best": value_best,
+           "ms_per_step": main_res["ms_per_step"], "ms_per_step_min": main_res["min"]["ms_per_step"], "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
            "dtype": "bf16", "data": "synthetic N(0,1) q/k/v/dO from a seeded device generator, random, no weights",
            "config": {"workload": {"c2": "causal 32k (config 2), forward", "c3": "strided 128k (config 3), forward+backward",
                                    "c4": "global+local 128k (config 4), forward+backward",
@@ -681,19 +779,22 @@ def main():
                       "seed": 0, "batch": 1, "heads": HEADS, "head_dim": 128, "block": BLOCK, "tile": 128,
                       "seq_q": int(workload_mask(a.workload).shape[0]) * BLOCK,
                       "seq_kv": int(workload_mask(a.workload).shape[1]) * BLOCK},
-           "frac_of_bf16_mfma_peak": value / peak, "peak_tflops": peak, "detail": main_res,
+           "frac_of_bf16_mfma_peak": value / peak, "frac_of_measured_mfma_ceiling": value / MEASURED_MFMA_CEILING[0],
+           "peak_tflops": peak, "detail": main_res,
            "fwd_frac_of_peak": main_res["fwd_tflops"] / peak, "roofline": roof, "rooflines": roofs, "extra": extra}
     if not a.no_extra:
         out["mask_builder"] = run_mask_builder(a.workload if a.workload != "c5" else "c3", 20)
         log(json.dumps(out["mask_builder"]))
         out["cols_gather"] = run_cols_gather(10)
         log(json.dumps(out["cols_gather"]))
+        torch.cuda.empty_cache()
+        out["grad_accumulate"] = run_grad_accumulate(10)
+        log(json.dumps(out["grad_accumulate"]))
         if a.workload != "c5":
             torch.cuda.empty_cache()
             out["power"] = run_power(a.workload)
             log(json.dumps(out["power"]))
-    out["mfma_probe"] = probe_mfma(peak)
-    log(json.dumps(out["mfma_probe"]))
+    out["mfma_probe"] = mfma_probe
     if not a.no_cpu:
         out["cpu_baseline"] = cpu_baseline()
         out["parity"] = out["cpu_baseline"]["parity"]          # the same object, at the top level too

@@ -6,6 +6,10 @@
 //                      follows the power drawn and the matrix pipe's power follows the bit
 //                      activity of its operands, so random operands give the practical ceiling
 //                      of any bf16 MFMA kernel fed with ordinary data.
+//   bench_probe_mfma_rotating / bench_probe_mfma16_rotating: the same with operands that change on every
+//                      instruction, for v_mfma_f32_32x32x16_bf16 and v_mfma_f32_16x16x32_bf16; with 256 or 512
+//                      workgroups of 4 waves (1 or 2 waves per SIMD) they give the device's ceiling rather than
+//                      one instruction's at one occupancy.
 //   bench_stream_mix   n_src streams read and one written with 16-byte accesses, the access
 //                      shape of the merge kernel: the device's rate for that read:write mix.
 //   bench_atomic_rate  device-wide rate of L2 atomics (fp32 add, u32 add, f64 add) and of plain dword
@@ -69,6 +73,34 @@ __global__ __launch_bounds__(256) void probe_mfma_rot_kernel(const u32x4* in, fl
   for (int i = 0; i < 4; ++i)
 #pragma unroll
     for (int j = 0; j < 16; ++j) s += c[i][j];
+  out[blockIdx.x * 256 + threadIdx.x] = s;
+}
+
+// The other dense bf16 instruction, v_mfma_f32_16x16x32_bf16 (16384 flop, 4 accumulator registers), with
+// rotating operands: 8 independent accumulators, 8 A x 8 B fragments cycled.
+typedef __attribute__((ext_vector_type(4))) float f32x4;
+__global__ __launch_bounds__(256) void probe_mfma16_rot_kernel(const u32x4* in, float* out, int iters) {
+  bf16x8 a[8], b[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    const u32x4 ra = in[(2 * i) * 256 + threadIdx.x], rb = in[(2 * i + 1) * 256 + threadIdx.x];
+    __builtin_memcpy(&a[i], &ra, 16);
+    __builtin_memcpy(&b[i], &rb, 16);
+  }
+  f32x4 c[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) c[i] = f32x4{0};
+  for (int it = 0; it < iters; it += 8) {
+#pragma unroll
+    for (int u = 0; u < 8; ++u)
+#pragma unroll
+      for (int i = 0; i < 8; ++i) c[i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[(u + i) & 7], b[(u + 3 * i) & 7], c[i], 0, 0, 0);
+  }
+  float s = 0.f;
+#pragma unroll
+  for (int i = 0; i < 8; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) s += c[i][j];
   out[blockIdx.x * 256 + threadIdx.x] = s;
 }
 
@@ -200,6 +232,17 @@ extern "C" int bench_probe_mfma_rotating(const void* operands, float* out, int n
   if (n_blocks <= 0 || iters <= 0) return -2;
   if (reinterpret_cast<uintptr_t>(operands) & 15) return -4;
   hipLaunchKernelGGL(probe_mfma_rot_kernel, dim3(n_blocks), dim3(256), 0, (hipStream_t)stream,
+                     (const u32x4*)operands, out, iters);
+  return hipGetLastError() == hipSuccess ? 0 : -6;
+}
+
+// Same operand layout as bench_probe_mfma_rotating; every thread issues 8 x iters (rounded up to a multiple
+// of 8) v_mfma_f32_16x16x32_bf16.
+extern "C" int bench_probe_mfma16_rotating(const void* operands, float* out, int n_blocks, int iters, void* stream) {
+  if (!operands || !out) return -1;
+  if (n_blocks <= 0 || iters <= 0) return -2;
+  if (reinterpret_cast<uintptr_t>(operands) & 15) return -4;
+  hipLaunchKernelGGL(probe_mfma16_rot_kernel, dim3(n_blocks), dim3(256), 0, (hipStream_t)stream,
                      (const u32x4*)operands, out, iters);
   return hipGetLastError() == hipSuccess ? 0 : -6;
 }

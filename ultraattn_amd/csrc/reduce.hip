@@ -12,7 +12,7 @@
 namespace ua {
 
 constexpr int kRedThreads = 256;
-constexpr int kRedBlocks = 8192;         // grid cap: 32 workgroups per CU, grid-stride beyond
+constexpr int kRedBlocks = 8192;         // grid cap of the sum: 32 workgroups per CU, grid-stride beyond
 
 __device__ __forceinline__ void unpack8(const u32x4 r, float (&x)[8]) {
 #pragma unroll
@@ -30,24 +30,44 @@ __device__ __forceinline__ bf16x8 pack8(const float (&x)[8]) {
 // mode 2: out  = bf16(float(out) + partial)                     (no fp32 accumulator)
 template <int kMode>
 __global__ __launch_bounds__(kRedThreads) void grad_accumulate_kernel(float* acc, const bf16* partial, bf16* out, int64_t n_chunks) {
-  for (int64_t c = (int64_t)blockIdx.x * kRedThreads + threadIdx.x; c < n_chunks; c += (int64_t)gridDim.x * kRedThreads) {
-    float x[8], y[8];
-    unpack8(__builtin_nontemporal_load(reinterpret_cast<const u32x4*>(partial) + c), y);
-    if (kMode == 0) {
-      const f32x4 a = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(acc) + 2 * c);
-      const f32x4 b = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(acc) + 2 * c + 1);
+  // kVec chunks of 8 elements per thread and step, every load of the step issued before the first use
+  constexpr int kVec = 4;
+  const int64_t stride = (int64_t)gridDim.x * kRedThreads * kVec;
+  for (int64_t c0 = (int64_t)blockIdx.x * kRedThreads * kVec + threadIdx.x; c0 < n_chunks; c0 += stride) {
+    u32x4 py[kVec], po[kVec];
+    f32x4 a0[kVec], a1[kVec];
 #pragma unroll
-      for (int j = 0; j < 4; ++j) { x[j] = a[j]; x[4 + j] = b[j]; }
-    } else {
-      unpack8(__builtin_nontemporal_load(reinterpret_cast<const u32x4*>(out) + c), x);
+    for (int u = 0; u < kVec; ++u) {
+      const int64_t c = c0 + u * kRedThreads;
+      if (c >= n_chunks) break;
+      py[u] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(partial) + c);
+      if (kMode == 0) {
+        a0[u] = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(acc) + 2 * c);
+        a1[u] = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(acc) + 2 * c + 1);
+      } else {
+        po[u] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(out) + c);
+      }
     }
 #pragma unroll
-    for (int j = 0; j < 8; ++j) x[j] += y[j];
-    if (kMode != 2) {
-      __builtin_nontemporal_store(f32x4{x[0], x[1], x[2], x[3]}, reinterpret_cast<f32x4*>(acc) + 2 * c);
-      __builtin_nontemporal_store(f32x4{x[4], x[5], x[6], x[7]}, reinterpret_cast<f32x4*>(acc) + 2 * c + 1);
+    for (int u = 0; u < kVec; ++u) {
+      const int64_t c = c0 + u * kRedThreads;
+      if (c >= n_chunks) break;
+      float x[8], y[8];
+      unpack8(py[u], y);
+      if (kMode == 0) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) { x[j] = a0[u][j]; x[4 + j] = a1[u][j]; }
+      } else {
+        unpack8(po[u], x);
+      }
+#pragma unroll
+      for (int j = 0; j < 8; ++j) x[j] += y[j];
+      if (kMode != 2) {
+        __builtin_nontemporal_store(f32x4{x[0], x[1], x[2], x[3]}, reinterpret_cast<f32x4*>(acc) + 2 * c);
+        __builtin_nontemporal_store(f32x4{x[4], x[5], x[6], x[7]}, reinterpret_cast<f32x4*>(acc) + 2 * c + 1);
+      }
+      if (out) __builtin_nontemporal_store(pack8(x), reinterpret_cast<bf16x8*>(out) + c);
     }
-    if (out) __builtin_nontemporal_store(pack8(x), reinterpret_cast<bf16x8*>(out) + c);
   }
 }
 
@@ -114,7 +134,7 @@ extern "C" int ua_grad_accumulate(float* acc, const void* partial, void* out, in
   if (n % 8 != 0 || !aligned16(partial) || (acc && !aligned16(acc)) || (out && !aligned16(out))) return UA_ERR_ALIGN;
   if (int rc = check_device()) return rc;
   const int64_t n_chunks = n / 8;
-  const int blocks = (int)std::min<int64_t>((n_chunks + kRedThreads - 1) / kRedThreads, kRedBlocks);
+  const int blocks = (int)std::min<int64_t>((n_chunks + 4 * kRedThreads - 1) / (4 * kRedThreads), 4 * kRedBlocks);
   hipStream_t st = (hipStream_t)stream;
   if (!acc)               hipLaunchKernelGGL(grad_accumulate_kernel<2>, dim3(blocks), dim3(kRedThreads), 0, st, acc, (const bf16*)partial, (bf16*)out, n_chunks);
   else if (init_from_out) hipLaunchKernelGGL(grad_accumulate_kernel<1>, dim3(blocks), dim3(kRedThreads), 0, st, acc, (const bf16*)partial, (bf16*)out, n_chunks);
