@@ -380,6 +380,65 @@ def run_cols_gather(steps):
             "shape": "[4, 2, 1, 32768, 32, 128] -> [2, 1, 131072, 32, 128] bf16, read + write"}
 
 
+def run_dense_split(steps):
+    """A dense rectangle with few tile lines (Sq=1024, Skv=4096, one head: 8 query tiles x 32 key tiles)
+    through the flash-attn call signature: the library cuts the walks into parts that fill the device
+    (forward: partial (O, LSE) + merge; backward: fp32 partial gradients + one sum).  Device time per
+    call from a HIP graph replay, next to the same entry points run unsplit (no workspace)."""
+    import torch
+    from ultraattn_amd import _lib, ops
+    from ultraattn_amd.flash_attn_interface import _flash_attn_backward, _flash_attn_forward
+    dev = "cuda:0"
+    sq, sk = 1024, 4096
+    g = torch.Generator(device=dev).manual_seed(0)
+    mk = lambda n: torch.randn(1, n, 1, 128, device=dev, dtype=torch.float32, generator=g).to(torch.bfloat16)
+    q, k, v, do = mk(sq), mk(sk), mk(sk), mk(sq)
+    o, dq, dk, dv = torch.empty_like(q), torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+    lse = _flash_attn_forward(q, k, v, 0.0, SCALE, causal=False, out=o)[5]
+    delta = ops.softmax_delta(o, do)
+    lib = _lib.load()
+    s3 = _lib.strides3
+
+    def unsplit_fwd():
+        st = torch.cuda.current_stream().cuda_stream
+        _lib.check(lib.ua_dense_fwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), lse.data_ptr(), 1, 1, sq, sk, 128,
+                                    s3(q), s3(k), s3(v), s3(o), SCALE, 0, None, 0, st), "ua_dense_fwd")
+
+    def unsplit_bwd():
+        st = torch.cuda.current_stream().cuda_stream
+        _lib.check(lib.ua_dense_bwd(do.data_ptr(), q.data_ptr(), k.data_ptr(), v.data_ptr(), lse.data_ptr(), delta.data_ptr(),
+                                    dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), 1, 1, sq, sk, 128, s3(q), s3(k), s3(v), s3(do),
+                                    s3(dq), s3(dk), s3(dv), SCALE, 0, None, 0, st), "ua_dense_bwd")
+    runs = {"fwd_split_us": lambda: _flash_attn_forward(q, k, v, 0.0, SCALE, causal=False, out=o),
+            "fwd_unsplit_us": unsplit_fwd,
+            "bwd_split_us": lambda: _flash_attn_backward(do, q, k, v, o, lse, dq, dk, dv, 0.0, SCALE, False, softmax_d=delta),
+            "bwd_unsplit_us": unsplit_bwd}
+    res = {"shape": "Sq=1024 Skv=4096 Nh=1 d=128 bf16, not causal (8 x 32 tiles)"}
+    for key, fn in runs.items():
+        fn()
+        torch.cuda.synchronize()
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=side):
+            for _ in range(steps):
+                fn()
+        graph.replay()
+        torch.cuda.synchronize()
+        best = float("inf")
+        for _ in range(REPEATS):
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            graph.replay()
+            e1.record()
+            torch.cuda.synchronize()
+            best = min(best, e0.elapsed_time(e1) / steps * 1e3)
+        res[key] = best
+    res["reference_h800_us"] = {"fwd": 23.392, "bwd": 86.88,
+                                "source": "prof_data/fit/time_g40_m2_flash_all.json, key [1024, 1, 1, 128, \"1/4\", false]"}
+    return res
+
+
 class PowerSampler:
     """Samples the socket power and the shader clock with `amd-smi metric -p -c` from a host thread
     while the GPU works (nothing is sampled inside the timed step loop of the benchmark)."""
@@ -790,6 +849,8 @@ def main():
         torch.cuda.empty_cache()
         out["grad_accumulate"] = run_grad_accumulate(10)
         log(json.dumps(out["grad_accumulate"]))
+        out["dense_split"] = run_dense_split(20)
+        log(json.dumps(out["dense_split"]))
         if a.workload != "c5":
             torch.cuda.empty_cache()
             out["power"] = run_power(a.workload)

@@ -79,6 +79,34 @@ def test_split_rectangles_match_the_oracle_and_the_unsplit_run(lib, sq, sk, nh, 
         assert max_abs(got, unsplit.cpu()) <= ATOL_O / 2
 
 
+@pytest.mark.parametrize("causal", [False, True])
+def test_split_with_batch_and_strided_views(lib, causal):
+    """Batch > 1 and q / k / v / gradients as strided views of packed buffers (token stride 2 * Nh * 128):
+    the partials are laid out [part][batch, tokens, heads, 128] whatever the callers' strides."""
+    B, sq, sk, nh = 2, 256, 1280, 2
+    g = torch.Generator().manual_seed(17)
+    pack = lambda n: torch.randn(B, n, 2 * nh, 128, generator=g).to(torch.bfloat16)
+    qp, kp, vp, dop = pack(sq), pack(sk), pack(sk), pack(sq)
+    q, k, v, do = qp[:, :, 0::2], kp[:, :, 1::2], vp[:, :, 0::2], dop[:, :, 1::2]
+    assert lib.ua_dense_workspace_bytes(B, nh, sq, sk, 0) > 0 and lib.ua_dense_workspace_bytes(B, nh, sq, sk, 1) > 0
+    dev = lambda t: t.to(DEV)
+    qd, kd, vd, dod = dev(qp)[:, :, 0::2], dev(kp)[:, :, 1::2], dev(vp)[:, :, 0::2], dev(dop)[:, :, 1::2]
+    res = _flash_attn_forward(qd, kd, vd, 0.0, SCALE, causal=causal)
+    O, lse = res[0], res[5]
+    gbuf = torch.zeros(B, sk, 2 * nh, 128, dtype=torch.bfloat16, device=DEV)
+    dk, dv = gbuf[:, :, 0::2], gbuf[:, :, 1::2]                    # [dK | dV] interleaved by head: strided outputs
+    dq = torch.empty_like(O)
+    _flash_attn_backward(dod, qd, kd, vd, O, lse, dq, dk, dv, 0.0, SCALE, causal)
+    torch.cuda.synchronize()
+    keep = keep_mask(sq, sk, causal)
+    for b in range(B):
+        sl = lambda t: t[b:b + 1].contiguous()
+        ro, rl = ao.dense_fwd(sl(q), sl(k), sl(v), SCALE, keep)
+        rq, rk, rv = ao.dense_bwd_autograd(sl(q), sl(k), sl(v), sl(do), SCALE, keep)
+        assert max_abs(O[b:b + 1], ro) <= ATOL_O and lse_rel_err(lse[b:b + 1], rl) <= RTOL_LSE
+        assert max_abs(dq[b:b + 1], rq) <= ATOL_O and max_abs(dk[b:b + 1], rk) <= ATOL_O and max_abs(dv[b:b + 1], rv) <= ATOL_O
+
+
 def test_dense_equals_the_tile_list_of_the_same_rectangle(lib):
     """List-free enumeration = the tile list that the block-mask builder gives for the same rectangle
     (bit for bit when nothing is split: same tiles in the same order)."""
