@@ -52,6 +52,9 @@ class TileList:
         import torch
         key = str(torch.device(device))
         if key not in self._dev:
+            if torch.cuda.is_current_stream_capturing():
+                # the staging buffers are released once the copies are done: a graph must not replay them
+                raise RuntimeError("TileList.on(device) must be called once before the stream is captured into a graph")
             # staged through pinned host memory and copied on the current stream without a host
             # synchronisation; the flag arrays are padded to a multiple of 4 bytes (the kernels read
             # them one aligned 32-bit word at a time)
@@ -71,7 +74,7 @@ class TileList:
             return dev
         dev = self._dev[key]
         ready = dev.get("_ready")
-        if ready is not None:
+        if ready is not None and not torch.cuda.is_current_stream_capturing():
             if ready.query():
                 dev["_ready"] = None
                 dev["_pinned"] = None
