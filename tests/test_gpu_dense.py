@@ -107,6 +107,34 @@ def test_split_with_batch_and_strided_views(lib, causal):
         assert max_abs(dq[b:b + 1], rq) <= ATOL_O and max_abs(dk[b:b + 1], rk) <= ATOL_O and max_abs(dv[b:b + 1], rv) <= ATOL_O
 
 
+@pytest.mark.parametrize("sq,sk,nh,causal", [(8192, 8192, 1, True), (4096, 16384, 1, False), (16384, 2048, 2, False)])
+def test_large_split_rectangles_equal_the_unsplit_run(lib, sq, sk, nh, causal):
+    """The reference planner's low-parallelism keys at their real sizes (one or two heads, thousands of
+    tokens: up to 16 parts per walk): split and unsplit runs of the same entry points agree to the
+    rounding of one bf16 result, and sampled rows agree with the oracle."""
+    g = torch.Generator(device=DEV).manual_seed(sq + sk)
+    mk = lambda n: torch.randn(1, n, nh, 128, device=DEV, dtype=torch.float32, generator=g).to(torch.bfloat16)
+    q, k, v, do = mk(sq), mk(sk), mk(sk), mk(sq)
+    assert lib.ua_dense_workspace_bytes(1, nh, sq, sk, 0) > 0 or lib.ua_dense_workspace_bytes(1, nh, sq, sk, 1) > 0
+    uo, ul, delta, udq, udk, udv = dense_unsplit(lib, q, k, v, do, causal)
+    res = _flash_attn_forward(q, k, v, 0.0, SCALE, causal=causal)
+    dq, dk, dv, _ = _flash_attn_backward(do, q, k, v, None, ul, None, None, None, 0.0, SCALE, causal, softmax_d=delta)
+    torch.cuda.synchronize()
+    assert max_abs(res[0], uo.cpu()) <= 8e-3 and lse_rel_err(res[5], ul.cpu()) <= 1e-5
+    for got, unsplit in ((dq, udq), (dk, udk), (dv, udv)):
+        assert max_abs(got, unsplit.cpu()) <= ATOL_O / 2
+    # sampled query rows against the dense formula (fp32 on the device, one head)
+    rows = torch.tensor([0, 1, 127, 128, sq // 2 + 5, sq - 129, sq - 1])
+    qs = q[0, rows, 0].float()
+    sc = (qs @ k[0, :, 0].float().T) * SCALE
+    if causal:
+        sc = sc.masked_fill(torch.arange(sk, device=DEV)[None, :] > rows.to(DEV)[:, None] + (sk - sq), float("-inf"))
+    want_lse = torch.logsumexp(sc, -1)
+    want_o = torch.softmax(sc, -1) @ v[0, :, 0].float()
+    assert (res[0][0, rows, 0].float() - want_o).abs().max().item() <= ATOL_O
+    assert ((res[5][0, 0, rows] - want_lse).abs() / want_lse.abs().clamp_min(1)).max().item() <= RTOL_LSE
+
+
 def test_dense_equals_the_tile_list_of_the_same_rectangle(lib):
     """List-free enumeration = the tile list that the block-mask builder gives for the same rectangle
     (bit for bit when nothing is split: same tiles in the same order)."""

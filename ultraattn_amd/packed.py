@@ -260,7 +260,7 @@ def create_buf_dict(q_shape, k_shape, fob: int, tensor_buf: torch.Tensor, comp_k
     if len(batch_degrees) != 2:
         raise ValueError(f"Invalid batch_degrees: {batch_degrees}")
     bs, Sq, Nh, D = q_shape
-    Skv = k_shape[1]
+    Skv, Nhg = k_shape[1], k_shape[2]          # the reference sizes the column packs with the K/V head count (Nhg)
     row_in = (lambda buf, n: InputRowFwd(buf, _scaled(q_shape, n))) if fob == 0 else \
         (lambda buf, n: InputRowBwd(buf, _scaled(q_shape, n), lse_slots=lse_slots))
     col_in = lambda buf, n: InputColFwd(buf, _scaled(k_shape, n))
@@ -291,9 +291,9 @@ def create_buf_dict(q_shape, k_shape, fob: int, tensor_buf: torch.Tensor, comp_k
     X, Y = fused_xy
     sq, skv = Sq * batch_degrees[0], Skv * batch_degrees[1]
     ir_nelems = bs * sq * Nh * (D if fob == 0 else 2 * D + 2 + lse_slots)
-    ic_nelems = bs * skv * Nh * 2 * D
+    ic_nelems = bs * skv * Nhg * 2 * D
     or_nelems = bs * sq * Nh * D
-    oc_nelems = 0 if fob == 0 else bs * skv * Nh * 2 * D
+    oc_nelems = 0 if fob == 0 else bs * skv * Nhg * 2 * D
     ir_tot, ic_tot, or_tot, oc_tot = ir_nelems * X, ic_nelems * Y, or_nelems * X, oc_nelems * Y
     end = ir_tot + ic_tot + or_tot + oc_tot
     buf = _take(tensor_buf, 0, end + (ir_tot if fob == 1 else 0))
