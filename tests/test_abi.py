@@ -113,6 +113,36 @@ def test_argument_checks_without_gpu(lib):
     assert lib.ua_strerror(-99) == b"unknown error code"
 
 
+def test_dense_entry_points_without_gpu(lib):
+    """Argument checks of ua_dense_fwd / ua_dense_bwd and the split policy behind
+    ua_dense_workspace_bytes (pure host arithmetic): a launch that fills the device or a short walk
+    never splits; else enough parts for ~2 workgroups per CU, at least two tiles each, at most 16."""
+    s = (ctypes.c_int64 * 3)(128 * 128, 128, 128)
+    buf = np.zeros(64, np.uint8).ctypes.data // 16 * 16 + 16
+    assert lib.ua_dense_fwd(None, buf, buf, buf, buf, 1, 1, 128, 128, 128, s, s, s, s, 0.1, 0, None, 0, None) == -1
+    assert lib.ua_dense_fwd(buf, buf, buf, buf, buf, 1, 1, 100, 128, 128, s, s, s, s, 0.1, 0, None, 0, None) == -2
+    assert lib.ua_dense_fwd(buf, buf, buf, buf, buf, 1, 1, 128, 0, 128, s, s, s, s, 0.1, 0, None, 0, None) == -2
+    assert lib.ua_dense_fwd(buf, buf, buf, buf, buf, 1, 1, 128, 128, 64, s, s, s, s, 0.1, 0, None, 0, None) == -3
+    assert lib.ua_dense_fwd(buf + 2, buf, buf, buf, buf, 1, 1, 128, 128, 128, s, s, s, s, 0.1, 0, None, 0, None) == -4
+    bwd = lambda *a: lib.ua_dense_bwd(*a, 1, 1, 128, 128, 128, s, s, s, s, s, s, s, 0.1, 1, None, 0, None)
+    assert bwd(buf, buf, buf, buf, buf, buf, None, buf, buf) == -1
+    assert bwd(buf, buf, buf, buf, None, buf, buf, buf, buf) == -1
+    assert lib.ua_dense_bwd(buf, buf, buf, buf, buf, buf, buf, buf, buf, 1, 1, 128, 130, 128, s, s, s, s, s, s, s, 0.1, 1,
+                            None, 0, None) == -2
+    ws = lib.ua_dense_workspace_bytes
+    assert ws(1, 32, 131072, 131072, 0) == 0 and ws(1, 32, 131072, 131072, 1) == 0       # 32768 workgroups
+    assert ws(1, 1, 256, 256, 0) == 0                                                  # 2 x 2 tiles: walks too short
+    assert ws(1, 1, 1000, 4096, 0) == 0 and ws(0, 1, 1024, 4096, 0) == 0                # nothing to size
+    al = lambda x: (x + 255) // 256 * 256
+    # Sq=1024, Skv=4096, one head: 8 query tiles, 32 key tiles -> min(16, ceil(512/8), 32/2) = 16 parts
+    assert ws(1, 1, 1024, 4096, 0) == 16 * (al(1024 * 128 * 2) + al(1024 * 4))
+    # backward: dQ 16 parts of fp32 [1024, 128]; dK, dV: 32 key tiles x 2 -> ceil(512/64) = 8, min(8, 16, 8/2) = 4 parts
+    assert ws(1, 1, 1024, 4096, 1) == 16 * al(1024 * 128 * 4) + 4 * 2 * al(4096 * 128 * 4)
+    # 32 heads x 8 query tiles = 256 workgroups < 384 -> ceil(512/256) = 2 parts
+    assert ws(1, 32, 1024, 4096, 0) == 2 * (al(32 * 1024 * 128 * 2) + al(32 * 1024 * 4))
+    assert ws(1, 32, 2048, 4096, 0) == 0                                               # 512 workgroups: full launch
+
+
 def test_missing_library_fails_loudly(monkeypatch, tmp_path):
     monkeypatch.setattr(_lib, "_lib", None)
     monkeypatch.setattr(_lib, "LIB_PATH", str(tmp_path / "nope.so"))

@@ -679,12 +679,12 @@ extern "C" int ua_dense_bwd(const void* dout, const void* q, const void* k, cons
   using namespace ua;
   if (seqlen_q <= 0 || seqlen_k <= 0 || seqlen_q % kTile || seqlen_k % kTile) return UA_ERR_SHAPE;
   const int n_qtiles = seqlen_q / kTile, n_ktiles = seqlen_k / kTile;
-  BwdParams p;
-  if (int rc = fill_common(p, q, k, v, dout, lse, delta, nullptr, nullptr, batch, n_heads, n_qtiles, n_ktiles, 0,
-                           head_dim, q_strides, k_strides, v_strides, do_strides, softmax_scale)) return rc;
   if (!dq || !dk || !dv || !dq_strides || !dk_strides || !dv_strides) return UA_ERR_NULL;
   if (!aligned16(dq) || !aligned16(dk) || !aligned16(dv) || !strides_ok(dq_strides) || !strides_ok(dk_strides) ||
       !strides_ok(dv_strides)) return UA_ERR_ALIGN;
+  BwdParams p;
+  if (int rc = fill_common(p, q, k, v, dout, lse, delta, nullptr, nullptr, batch, n_heads, n_qtiles, n_ktiles, 0,
+                           head_dim, q_strides, k_strides, v_strides, do_strides, softmax_scale)) return rc;
   hipStream_t st = (hipStream_t)stream;
   p.dense = 1; p.dense_causal = causal != 0; p.diag_off = n_ktiles - n_qtiles;
   const DenseSplit d = dense_split(batch, n_heads, n_qtiles, n_ktiles);
