@@ -17,8 +17,11 @@ from .ops import HEAD_DIM, _check_qkv, softmax_delta
 from .tilelist import TILE
 
 # (device index, stream handle) -> uint8 tensor holding the partial results of split calls.  Calls
-# on one stream run in order, so they can share it; it only ever grows.
+# on one stream run in order, so they can share it; it only ever grows.  At most _MAX_WORKSPACES are
+# kept (least recently used first out: stream handles come and go).
 _workspaces: Dict[Tuple[int, int], torch.Tensor] = {}
+_MAX_WORKSPACES = 16
+_captured = []             # workspaces that a captured graph may replay into: never released
 _initialised = set()
 
 
@@ -40,10 +43,14 @@ def _workspace(lib, q, k, backward: bool, stream: int):
     if need <= 0:
         return None, 0
     key = (q.device.index, stream)
-    ws = _workspaces.get(key)
+    ws = _workspaces.pop(key, None)
     if ws is None or ws.numel() < need:
         ws = torch.empty(need, dtype=torch.uint8, device=q.device)
-        _workspaces[key] = ws
+    _workspaces[key] = ws                      # most recently used last
+    while len(_workspaces) > _MAX_WORKSPACES:
+        _workspaces.pop(next(iter(_workspaces)))
+    if torch.cuda.is_current_stream_capturing() and not any(w is ws for w in _captured):
+        _captured.append(ws)                   # outlives its cache entry: the graph keeps writing to it
     return ws.data_ptr(), ws.numel()
 
 
