@@ -439,6 +439,59 @@ def run_dense_split(steps):
     return res
 
 
+def run_per_rectangle(name):
+    """What the single launch over a tile list replaces: the reference's executors run a device's
+    share as one dense flash-attention call per (row chunk, column chunk) rectangle and fold the
+    partial (O, LSE) pairs (orchestrated_attn_impl.py:348-349, ring_flash_attn/utils.py:78-99).  The
+    same kernels driven that way (BlockSparseExecutor.forward_per_rectangle: ua_dense_fwd +
+    ua_merge_update per rectangle), forward only: issued from Python, and as one HIP graph replay
+    (device time without the host's launch cost), next to the single launch."""
+    import torch
+    from ultraattn_amd.executor import BlockSparseExecutor
+    dev = "cuda:0"
+    mask = workload_mask(name)
+    g = torch.Generator(device=dev).manual_seed(0)
+    mk = lambda n: torch.randn(1, n * BLOCK, HEADS, 128, device=dev, dtype=torch.float32, generator=g).to(torch.bfloat16)
+    q, k, v = mk(mask.shape[0]), mk(mask.shape[1]), mk(mask.shape[1])
+    ex = BlockSparseExecutor(mask, BLOCK, softmax_scale=SCALE)
+    o1, l1 = ex.forward(q, k, v)
+    o2, l2 = ex.forward_per_rectangle(q, k, v)
+    torch.cuda.synchronize()
+    fin = torch.isfinite(l1)
+    res = {"workload": name, "rectangles": int((mask != 0).sum()),
+           "max_abs_o_vs_single_launch": (o1.float() - o2.float()).abs().max().item(),
+           "max_abs_lse_vs_single_launch": (l1[fin] - l2[fin]).abs().max().item()}
+
+    def timed(fn, n):
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(n):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) / n
+    res["single_launch_ms"] = timed(lambda: ex.forward(q, k, v, out=o1, lse=l1), 5)
+    t0 = time.perf_counter()
+    res["per_rectangle_eager_ms"] = timed(lambda: ex.forward_per_rectangle(q, k, v), 1)
+    res["per_rectangle_eager_wall_ms"] = (time.perf_counter() - t0) * 1e3
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        ex.forward_per_rectangle(q, k, v)
+    graph.replay()
+    torch.cuda.synchronize()
+    res["per_rectangle_graph_replay_ms"] = min(timed(graph.replay, 1) for _ in range(REPEATS))
+    # without the folding, as the reference's harness runs it (its reduce() is a stub)
+    res["per_rectangle_no_fold_ms"] = min(timed(lambda: ex.forward_per_rectangle(q, k, v, fold=False), 1) for _ in range(2))
+    F = fwd_flops(mask)
+    res["single_launch_tflops"] = F / res["single_launch_ms"] / 1e9
+    res["per_rectangle_graph_tflops"] = F / res["per_rectangle_graph_replay_ms"] / 1e9
+    res["speedup_vs_graph_replay"] = res["per_rectangle_graph_replay_ms"] / res["single_launch_ms"]
+    res["speedup_vs_no_fold"] = res["per_rectangle_no_fold_ms"] / res["single_launch_ms"]
+    return res
+
+
 class PowerSampler:
     """Samples the socket power and the shader clock with `amd-smi metric -p -c` from a host thread
     while the GPU works (nothing is sampled inside the timed step loop of the benchmark)."""
@@ -851,6 +904,10 @@ def main():
         log(json.dumps(out["grad_accumulate"]))
         out["dense_split"] = run_dense_split(20)
         log(json.dumps(out["dense_split"]))
+        if a.workload in ("c3", "c4"):
+            torch.cuda.empty_cache()
+            out["per_rectangle_baseline"] = run_per_rectangle(a.workload)
+            log(json.dumps(out["per_rectangle_baseline"]))
         if a.workload != "c5":
             torch.cuda.empty_cache()
             out["power"] = run_power(a.workload)

@@ -57,6 +57,24 @@ def test_schedule_table_and_kernel_tiles():
     assert (o0 == 0).all() and torch.isinf(l0).all()
 
 
+@pytest.mark.parametrize("make,chunk", [(lambda: masks.config_strided(8, 2, 4), 256), (lambda: masks.config_global_local(6, 1, 2), 128),
+                                        (lambda: masks.canonical_block_table(3), 128)])
+def test_one_dense_call_per_rectangle_equals_the_single_launch(make, chunk):
+    """The reference's way of running a device's share (a dense tile call per chunk pair, partials
+    folded with update_out_and_lse) and the single launch over the tile list give the same result."""
+    table = make()
+    q, k, v, _ = seeded_inputs(table, chunk, seed=21, nh=3)
+    qd, kd, vd = (t.to(DEV) for t in (q, k, v))
+    ex = BlockSparseExecutor(table, chunk, softmax_scale=SCALE)
+    o1, l1 = ex.forward(qd, kd, vd)
+    o2, l2 = ex.forward_per_rectangle(qd, kd, vd)
+    torch.cuda.synchronize()
+    keep = ao.element_mask(table, chunk)
+    ro, rl = ao.dense_fwd(q, k, v, SCALE, keep)
+    assert max_abs(o2, ro) <= ATOL_O and lse_rel_err(l2, rl) <= RTOL_LSE
+    assert max_abs(o2, o1.cpu()) <= 8e-3 and lse_rel_err(l2, l1.cpu()) <= 1e-5
+
+
 def test_kernels_run_in_place_on_packed_buffers():
     """Forward and backward straight on the packed row / column views, D filled in the pack."""
     table = masks.config_causal(2)

@@ -125,6 +125,36 @@ class BlockSparseExecutor:
                  for t, (po, pl) in zip(self.kernel_tiles, self._partials(q))]
         return merge_partials([p[0] for p in parts], [p[1] for p in parts], out=out, lse=lse)
 
+    def forward_per_rectangle(self, q, k, v, fold: bool = True):
+        """-> (out, lse) computed the way the reference's executors do it: one dense tile call per
+        non-empty chunk pair, in the row-major order of the kernel list
+        (``intra_attn_forward``'s loop, ``orchestrated_attn/orchestrated_attn_impl.py:348-349``; a
+        chunk is causal iff its type is CAUSAL, ``:91``), each partial ``(O, LSE)`` folded into the
+        row chunk's running result with ``update_out_and_lse(..., slice_=)``
+        (``ring_flash_attn/utils.py:78-99``, as ``hierarchy_attn/hierarchy_attn_impl.py:64-81`` does),
+        running output in fp32, running LSE ``[B, S, Nh, 1]``.  Same result as ``forward`` to the
+        parity bar; it exists to measure what the single launch over a tile list replaces, and as
+        a second, independent path through the kernels.  ``fold=False`` leaves the folding out, as
+        the reference's harness does (its ``reduce`` is ``pass``, ``orchestrated_attn/utils.py:119-134``):
+        every rectangle overwrites its row chunk, the result is the last rectangle's and only the
+        time means anything."""
+        from .flash_attn_interface import _flash_attn_forward
+        from .ops import update_out_and_lse
+        B, Sq, Nh, D = q.shape
+        c = self.chunk
+        scale = self.softmax_scale if self.softmax_scale is not None else D ** -0.5
+        out = torch.zeros(B, Sq, Nh, D, dtype=torch.float32, device=q.device)
+        lse = torch.full((B, Sq, Nh, 1), float("-inf"), dtype=torch.float32, device=q.device)
+        blk = torch.empty(B, c, Nh, D, dtype=q.dtype, device=q.device)
+        for r, row in enumerate(self.mask):
+            rows = slice(r * c, (r + 1) * c)
+            for col in np.nonzero(row)[0]:
+                cols = slice(int(col) * c, (int(col) + 1) * c)
+                res = _flash_attn_forward(q[:, rows], k[:, cols], v[:, cols], 0.0, scale, causal=bool(row[col] == CAUSAL), out=blk)
+                if fold:
+                    update_out_and_lse(out, lse, res[0], res[5], slice_=(slice(None), rows))
+        return out.to(q.dtype), lse.squeeze(-1).transpose(1, 2).contiguous()
+
     def backward(self, dout, q, k, v, out, lse, dq=None, dk=None, dv=None, softmax_d=None):
         """-> (dq, dk, dv).  ``lse`` (and ``softmax_d``) are the rows' GLOBAL statistics: when this
         device holds only part of a row's keys they are those of the merged result."""
