@@ -63,7 +63,7 @@ def test_one_dense_call_per_rectangle_equals_the_single_launch(make, chunk):
     """The reference's way of running a device's share (a dense tile call per chunk pair, partials
     folded with update_out_and_lse) and the single launch over the tile list give the same result."""
     table = make()
-    q, k, v, _ = seeded_inputs(table, chunk, seed=21, nh=3)
+    q, k, v, do = seeded_inputs(table, chunk, seed=21, nh=3)
     qd, kd, vd = (t.to(DEV) for t in (q, k, v))
     ex = BlockSparseExecutor(table, chunk, softmax_scale=SCALE)
     o1, l1 = ex.forward(qd, kd, vd)
@@ -73,6 +73,18 @@ def test_one_dense_call_per_rectangle_equals_the_single_launch(make, chunk):
     ro, rl = ao.dense_fwd(q, k, v, SCALE, keep)
     assert max_abs(o2, ro) <= ATOL_O and lse_rel_err(l2, rl) <= RTOL_LSE
     assert max_abs(o2, o1.cpu()) <= 8e-3 and lse_rel_err(l2, l1.cpu()) <= 1e-5
+    # backward: a dense call per rectangle with the rows' global statistics, fp32 running sums
+    dod = do.to(DEV)
+    delta = ops.softmax_delta(o1, dod)
+    g1 = ex.backward(dod, qd, kd, vd, None, l1, softmax_d=delta)
+    g2 = ex.backward_per_rectangle(dod, qd, kd, vd, l1, delta)
+    torch.cuda.synchronize()
+    want = ao.dense_bwd_autograd(q, k, v, do, SCALE, keep)
+    for a, b, w in zip(g1, g2, want):
+        # every partial is rounded to bf16 before it is added (as in the reference): the bar scales with
+        # the size of the gradients, which on these short rows reach several units
+        bar = ATOL_O * max(1.0, float(w.abs().max()))
+        assert max_abs(a, w) <= ATOL_O and max_abs(b, w) <= bar and max_abs(b, a.cpu()) <= bar
 
 
 def test_kernels_run_in_place_on_packed_buffers():

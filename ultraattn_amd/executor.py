@@ -155,6 +155,35 @@ class BlockSparseExecutor:
                     update_out_and_lse(out, lse, res[0], res[5], slice_=(slice(None), rows))
         return out.to(q.dtype), lse.squeeze(-1).transpose(1, 2).contiguous()
 
+    def backward_per_rectangle(self, dout, q, k, v, lse, softmax_d):
+        """-> (dq, dk, dv) the reference's way: one dense backward call per non-empty chunk pair
+        (``intra_attn_backward``'s loop, ``orchestrated_attn/orchestrated_attn_impl.py:554-620``) with
+        the rows' global ``lse`` and ``softmax_d``, every partial gradient added into an fp32 running
+        sum per row chunk (dQ) or column chunk (dK, dV) and cast once at the end
+        (``ring_flash_attn/ring_flash_attn.py:110-118, 135``), one ``ua_grad_accumulate`` per partial."""
+        from .flash_attn_interface import _flash_attn_backward
+        from .ops import grad_accumulate
+        B, Sq, Nh, D = q.shape
+        c = self.chunk
+        scale = self.softmax_scale if self.softmax_scale is not None else D ** -0.5
+        f32 = dict(dtype=torch.float32, device=q.device)
+        acc_q = [torch.zeros(B, c, Nh, D, **f32) for _ in range(self.mask.shape[0])]
+        acc_k = [torch.zeros(B, c, Nh, D, **f32) for _ in range(self.mask.shape[1])]
+        acc_v = [torch.zeros(B, c, Nh, D, **f32) for _ in range(self.mask.shape[1])]
+        gq, gk, gv = (torch.empty(B, c, Nh, D, dtype=q.dtype, device=q.device) for _ in range(3))
+        for r, row in enumerate(self.mask):
+            rows = slice(r * c, (r + 1) * c)
+            lse_r, d_r = lse[:, :, rows].contiguous(), softmax_d[:, :, rows].contiguous()
+            for col in np.nonzero(row)[0]:
+                cols = slice(int(col) * c, (int(col) + 1) * c)
+                _flash_attn_backward(dout[:, rows], q[:, rows], k[:, cols], v[:, cols], None, lse_r, gq, gk, gv, 0.0, scale,
+                                     bool(row[col] == CAUSAL), softmax_d=d_r)
+                grad_accumulate(gq, None, acc=acc_q[r])
+                grad_accumulate(gk, None, acc=acc_k[int(col)])
+                grad_accumulate(gv, None, acc=acc_v[int(col)])
+        cat = lambda parts: torch.cat([a.to(q.dtype) for a in parts], dim=1)
+        return cat(acc_q), cat(acc_k), cat(acc_v)
+
     def backward(self, dout, q, k, v, out, lse, dq=None, dk=None, dv=None, softmax_d=None):
         """-> (dq, dk, dv).  ``lse`` (and ``softmax_d``) are the rows' GLOBAL statistics: when this
         device holds only part of a row's keys they are those of the merged result."""
